@@ -192,6 +192,13 @@ MIXERS_SIGNATURES = {
     "aphro_experts_down_gemm": (I, [P, P, P, P, P, P, L, L, I, I, I, I, I, P]),
     "aphro_experts_combine": (I, [P, P, P, P, P, L, P, L, P, L, L, I, I, I, I, P]),
     "aphro_clamped_glu": (I, [P, P, L, L, I, F, F, I, P]),
+    "aphro_hashed_pair_embed": (I, [P, P, P, P, P, P, P, P, P, L, I, L, L, L, L, I, P]),
+    "aphro_token_state_write": (I, [P, P, P, P, P, I, P]),
+    "aphro_residual_add2_rms_norm": (I, [P, P, L, P, L, P, P, P, L, I, F, I, P]),
+    "aphro_latent_prep": (I, [P, P, L, P, L, I, I, P, P, P, P, P, P, P, F, L, I, I, I, I, F, I, P]),
+    "aphro_latent_attention_plain": (I, [P, L, L, P, L, L, P, L, L, P, P, I, L, I, P, P, P, P, F, L, I, I, I, I, F, I, P]),
+    "aphro_sigmoid_gate_mul": (I, [P, L, P, L, P, L, L, I, I, P]),
+    "aphro_experts_route_grouped": (I, [P, P, P, L, I, I, I, I, I, F, P]),
 }
 
 OK = 0

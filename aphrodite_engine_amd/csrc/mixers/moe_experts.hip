@@ -14,8 +14,10 @@ namespace aphro {
 
 constexpr int MOE_BM = 16;
 
-// g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha g) * (u + 1)
+// limit > 0:  g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha g) * (u + 1)
+// limit <= 0: the plain gated form gate * sigmoid(alpha gate) * up (alpha 1: silu)
 __device__ __forceinline__ float clamped_glu_f(float gate, float up, float limit, float alpha) {
+  if (limit <= 0.f) return gate * sigmoid_f(alpha * gate) * up;
   const float g = fminf(gate, limit);
   const float u = fminf(fmaxf(up, -limit), limit);
   return g * sigmoid_f(alpha * g) * (u + 1.0f);
@@ -74,6 +76,106 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ id
       if (live) {
         ids[t * top + k] = bi;
         weights[t * top + k] = s[bi];
+      }
+      ch[bi] = -INFINITY;
+    }
+    __syncthreads();
+  }
+}
+
+// Sigmoid router with a choice limited to the best groups of neighbouring experts; one wave per token.  s = sigmoid(z); a
+// group's score is the sum of its `group_top` largest s; only experts of the `keep` best groups can be chosen; the `top`
+// largest s among those are chosen and weighted by s * scale (not renormalised).  Ties go to the lower index.
+__global__ __launch_bounds__(256) void moe_route_grouped_kernel(int32_t* __restrict__ ids, float* __restrict__ weights,
+                                                                const float* __restrict__ z, int64_t num_tokens, int experts,
+                                                                int top, int groups, int keep, int group_top, float scale) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* s = lds + (size_t)wave * (2 * experts + groups);
+  float* ch = s + experts;
+  float* gsc = ch + experts;
+  const int64_t tt = (int64_t)blockIdx.x * 4 + wave;
+  const bool live = tt < num_tokens;
+  const int64_t t = live ? tt : num_tokens - 1;
+  const float* zr = z + t * experts;
+  const int gsz = experts / groups;
+  for (int i = lane; i < experts; i += 64) {
+    const float p = sigmoid_f(zr[i]);
+    s[i] = p;
+    ch[i] = -INFINITY;                        // not allowed until its group is kept
+  }
+  __syncthreads();
+  for (int g = lane; g < groups; g += 64) {   // sum of the group's group_top largest, by repeated maximum
+    float sum = 0.f;
+    float last = INFINITY;
+    int last_i = -1;
+    for (int k = 0; k < group_top && k < gsz; ++k) {
+      float bv = -INFINITY;
+      int bi = -1;
+      for (int i = 0; i < gsz; ++i) {
+        const float v = s[g * gsz + i];
+        const bool below = v < last || (v == last && i > last_i);      // after the previous pick in (value desc, index asc)
+        if (below && v > bv) {
+          bv = v;
+          bi = i;
+        }
+      }
+      if (bi < 0) break;
+      sum += bv;
+      last = bv;
+      last_i = bi;
+    }
+    gsc[g] = sum;
+  }
+  __syncthreads();
+  for (int k = 0; k < keep; ++k) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int g = lane; g < groups; g += 64) {
+      const float v = gsc[g];
+      if (v > bv) {
+        bv = v;
+        bi = g;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (bi >= groups) bi = 0;
+    for (int i = lane; i < gsz; i += 64) ch[bi * gsz + i] = s[bi * gsz + i];
+    if (lane == 0) gsc[bi] = -INFINITY;
+    __syncthreads();
+  }
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = lane; i < experts; i += 64) {
+      const float v = ch[i];
+      if (v > bv) {
+        bv = v;
+        bi = i;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (bi >= experts) bi = 0;
+    if (lane == 0) {
+      if (live) {
+        ids[t * top + k] = bi;
+        weights[t * top + k] = s[bi] * scale;
       }
       ch[bi] = -INFINITY;
     }
@@ -424,6 +526,19 @@ extern "C" int aphro_experts_route(int32_t* ids, float* weights, const float* ro
               "moe_route: %d router outputs (<= 2048), top %d", outputs, top);
   hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((num_tokens + 3) / 4)), dim3(256), (size_t)8 * outputs * sizeof(float),
                      (hipStream_t)stream, ids, weights, router_out, correction, num_tokens, outputs, top);
+  APHRO_LAUNCH_CHECK();
+  return APHRO_OK;
+}
+
+extern "C" int aphro_experts_route_grouped(int32_t* ids, float* weights, const float* router_out, int64_t num_tokens, int experts,
+                                           int top, int groups, int keep, int group_top, float scale, void* stream) {
+  if (num_tokens == 0) return APHRO_OK;
+  APHRO_CHECK(ids && weights && router_out && experts > 0 && experts <= 2048 && groups > 0 && experts % groups == 0 && keep > 0 &&
+                  keep <= groups && group_top > 0 && top > 0 && top <= keep * (experts / groups),
+              "moe_route_grouped: %d experts (<= 2048) in %d groups of which %d are kept, top %d", experts, groups, keep, top);
+  hipLaunchKernelGGL(moe_route_grouped_kernel, dim3((unsigned)((num_tokens + 3) / 4)), dim3(256),
+                     (size_t)4 * (2 * experts + groups) * sizeof(float), (hipStream_t)stream, ids, weights, router_out, num_tokens,
+                     experts, top, groups, keep, group_top, scale);
   APHRO_LAUNCH_CHECK();
   return APHRO_OK;
 }

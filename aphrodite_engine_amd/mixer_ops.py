@@ -482,3 +482,159 @@ def clamped_glu(x: torch.Tensor, d: int, limit: float, alpha: float) -> torch.Te
     check(_lib.mixers_lib().aphro_clamped_glu(out.data_ptr(), x.data_ptr(), x.stride(0) if x.shape[0] > 1 else max(x.stride(0), 2 * d),
                                               x.shape[0], d, float(limit), float(alpha), _dt(x), _stream()), "clamped_glu")
     return out
+
+
+# ---- sublayers side by side, hashed token-pair embedding, attention through a low-rank latent ------------------------------------
+def hashed_pair_embed(table: torch.Tensor, pair_table: torch.Tensor, ids: torch.Tensor, token_state: torch.Tensor,
+                      state_slots: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor,
+                      seq_of_token: torch.Tensor, mul_prev: int, mul_cur: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 rows ``table[id] + pair_table[(previous * mul_prev + id * mul_cur) mod buckets]`` (row ``buckets`` for a sequence's
+    first token; pair_table has buckets + 1 rows).  ``token_state`` int32 [slots] holds every live request's last token: it is
+    read for a segment's first row and advanced to the segment's last token."""
+    _cuda(table, pair_table, ids, token_state, state_slots, q_start, q_len, ctx_len, seq_of_token, out)
+    T, S, W = ids.shape[0], q_start.numel(), table.shape[1]
+    _need(table.dim() == 2 and table.is_contiguous() and pair_table.dim() == 2 and pair_table.is_contiguous()
+          and pair_table.shape[1] == W and pair_table.shape[0] >= 2 and pair_table.dtype == table.dtype,
+          "hashed_pair_embed: table [vocab, width], pair_table [buckets + 1, width], one dtype")
+    _need(ids.dtype == torch.int64 and ids.dim() == 1 and ids.is_contiguous(), "hashed_pair_embed: ids int64 [T]")
+    _need(token_state.dtype == torch.int32 and token_state.dim() == 1 and token_state.is_contiguous(),
+          "hashed_pair_embed: token_state int32 [slots]")
+    for t, nm in ((state_slots, "state_slots"), (q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+        _i32(t, S, nm)
+    _i32(seq_of_token, T, "seq_of_token")
+    if out is None:
+        out = torch.empty(T, W, dtype=torch.float32, device=table.device)
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, W), "hashed_pair_embed: out fp32 [T, width]")
+    lib, st = _lib.mixers_lib(), _stream()
+    check(lib.aphro_hashed_pair_embed(out.data_ptr(), table.data_ptr(), pair_table.data_ptr(), ids.data_ptr(), token_state.data_ptr(),
+                                      state_slots.data_ptr(), q_start.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), T, W,
+                                      table.shape[0], pair_table.shape[0] - 1, int(mul_prev), int(mul_cur), _dt(table), st),
+          "hashed_pair_embed")
+    check(lib.aphro_token_state_write(token_state.data_ptr(), ids.data_ptr(), state_slots.data_ptr(), q_start.data_ptr(),
+                                      q_len.data_ptr(), S, st), "token_state_write")
+    return out
+
+
+def residual_add2_rms_norm(x: torch.Tensor, ya: Optional[torch.Tensor] = None, yb: Optional[torch.Tensor] = None,
+                           bias: Optional[torch.Tensor] = None, weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
+                           dtype: Optional[torch.dtype] = None, want_out: bool = True) -> Optional[torch.Tensor]:
+    """x += ya + yb + bias in place (fp32 [T, W]; each term optional), then returns rms_norm(x) * weight in the activation dtype
+    (``want_out`` False: the add alone)."""
+    T, W = x.shape
+    _cuda(x, ya, yb, bias, weight)
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "residual_add2_rms_norm: x is fp32, contiguous")
+    some = next((t for t in (ya, yb, weight, bias) if t is not None), None)
+    adt = dtype or (some.dtype if some is not None else None)
+    _need(adt in _DT, "residual_add2_rms_norm: the activation dtype is not given")
+    sa = sb = 0
+    if ya is not None:
+        _need(ya.dtype == adt and ya.shape[0] == T, "residual_add2_rms_norm: ya [T, W] of the activation dtype")
+        sa = _rows(ya, W, "residual_add2_rms_norm ya")
+    if yb is not None:
+        _need(yb.dtype == adt and yb.shape[0] == T, "residual_add2_rms_norm: yb [T, W] of the activation dtype")
+        sb = _rows(yb, W, "residual_add2_rms_norm yb")
+    for v in (bias, weight):
+        _need(v is None or (v.dtype == adt and v.numel() == W and v.is_contiguous()), "residual_add2_rms_norm: vectors [W] of the activation dtype")
+    out = torch.empty(T, W, dtype=adt, device=x.device) if want_out else None
+    check(_lib.mixers_lib().aphro_residual_add2_rms_norm(x.data_ptr(), _p(ya), sa, _p(yb), sb, _p(bias), _p(weight), _p(out), T, W,
+                                                         float(eps), _DT[adt], _stream()), "residual_add2_rms_norm")
+    return out
+
+
+def latent_prep(proj: torch.Tensor, q_at: int, q_rank: int, kv_at: int, kv_rank: int, rot_dim: int, rot_dims: int,
+                wq: Optional[torch.Tensor], wkv: torch.Tensor, cache: torch.Tensor, slot_mapping: torch.Tensor,
+                q_start: torch.Tensor, ctx_len: torch.Tensor, seq_of_token: torch.Tensor, inv_freq: Optional[torch.Tensor],
+                mscale: float, eps: float) -> Optional[torch.Tensor]:
+    """From the rows of one input product: the normed query latent [T, q_rank] (returned), and the cache row of every token --
+    its normed key/value latent and the shared key part rotated at the token's position -- written at ``slot_mapping``.
+    cache [blocks, block, kv_rank + rot_dim]."""
+    _cuda(proj, wq, wkv, cache, slot_mapping, q_start, ctx_len, seq_of_token, inv_freq)
+    T, S = proj.shape[0], q_start.numel()
+    _need(proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= max(q_at + q_rank, kv_at + kv_rank + rot_dim),
+          "latent_prep: proj rows hold the latents")
+    _need(cache.dim() == 3 and cache.is_contiguous() and cache.shape[2] == kv_rank + rot_dim and cache.dtype == proj.dtype,
+          "latent_prep: cache [blocks, block, kv_rank + rot_dim] of the activation dtype")
+    _need(wkv.dtype == proj.dtype and wkv.numel() == kv_rank and wkv.is_contiguous(), "latent_prep: wkv [kv_rank]")
+    _need(q_rank == 0 or (wq is not None and wq.dtype == proj.dtype and wq.numel() == q_rank and wq.is_contiguous()),
+          "latent_prep: wq [q_rank]")
+    _need(slot_mapping.dtype == torch.int64 and slot_mapping.numel() == T and slot_mapping.is_contiguous(), "latent_prep: slots int64 [T]")
+    _i32(q_start, S, "q_start")
+    _i32(ctx_len, S, "ctx_len")
+    _i32(seq_of_token, T, "seq_of_token")
+    _need(rot_dims == 0 or (inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2
+                            and inv_freq.is_contiguous()), "latent_prep: inv_freq fp32 [rot_dims / 2]")
+    cq = torch.empty(T, q_rank, dtype=proj.dtype, device=proj.device) if q_rank else None
+    stride = proj.stride(0) if T > 1 else max(proj.stride(0), proj.shape[1])
+    check(_lib.mixers_lib().aphro_latent_prep(_p(cq), cache.data_ptr(), cache.shape[0] * cache.shape[1], proj.data_ptr(), stride,
+                                              int(q_at), int(kv_at), _p(wq), wkv.data_ptr(), slot_mapping.data_ptr(),
+                                              q_start.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), _p(inv_freq),
+                                              float(mscale), T, int(q_rank), int(kv_rank), int(rot_dim), int(rot_dims), float(eps),
+                                              _dt(proj), _stream()), "latent_prep")
+    return cq
+
+
+def _head_view(t: torch.Tensor, T: int, heads: int, n: int, what: str):
+    """(token stride, head stride) of a [T, heads, n] view whose last axis is dense."""
+    _need(t.dim() == 3 and tuple(t.shape) == (T, heads, n) and (t.stride(2) == 1 or n == 1), f"{what}: [T, heads, {n}] with a dense last axis")
+    return t.stride(0), t.stride(1)
+
+
+def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: Optional[torch.Tensor], cache: torch.Tensor,
+                     block_tables: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor,
+                     seq_of_token: torch.Tensor, q_len_range, inv_freq: Optional[torch.Tensor], mscale: float, rot_dims: int,
+                     scale: float, max_kv_len: int = 0) -> None:
+    """Causal softmax attention of a batch of segments over latent cache rows [c | k_r] that all heads share.  q_lat
+    [T, heads, kv_rank] (every head's query carried into the latent), q_rot [T, heads, rot_dim] (raw: rotated here at the row's
+    position), out [T, heads, kv_rank] = sum_j p_ij c_j -- any strides over tokens and heads.  ``q_len_range`` (shortest, longest
+    segment) and ``max_kv_len`` (longest ctx_len + q_len), known on the host, choose the kernel and its work split."""
+    _cuda(out, q_lat, q_rot, cache, block_tables, q_start, q_len, ctx_len, seq_of_token, inv_freq)
+    T, H, R = q_lat.shape
+    nb, bs, D = cache.shape
+    P_ = D - R
+    S = q_start.numel()
+    _need(cache.is_contiguous() and cache.dtype == q_lat.dtype == out.dtype and P_ >= 0, "latent_attention: cache [blocks, block, rank + rot]")
+    os_, ohs = _head_view(out, T, H, R, "latent_attention out")
+    qs, qhs = _head_view(q_lat, T, H, R, "latent_attention q_lat")
+    rs = rhs = 0
+    if P_:
+        _need(q_rot is not None and q_rot.dtype == q_lat.dtype, "latent_attention: q_rot of the activation dtype")
+        rs, rhs = _head_view(q_rot, T, H, P_, "latent_attention q_rot")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] == S and block_tables.is_contiguous(),
+          "latent_attention: block_tables int32 [S, max_blocks]")
+    for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+        _i32(t, S, nm)
+    _i32(seq_of_token, T, "seq_of_token")
+    _need(rot_dims == 0 or (inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2
+                            and inv_freq.is_contiguous()), "latent_attention: inv_freq fp32 [rot_dims / 2]")
+    check(_lib.mixers_lib().aphro_latent_attention_plain(
+        out.data_ptr(), os_, ohs, q_lat.data_ptr(), qs, qhs, _p(q_rot), rs, rhs, cache.data_ptr(), block_tables.data_ptr(),
+        block_tables.shape[1], nb, bs, q_start.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), _p(inv_freq), float(mscale), T,
+        H, R, P_, int(rot_dims), float(scale), _dt(q_lat), _stream()), "latent_attention")
+
+
+def sigmoid_gate_mul(x: torch.Tensor, gate: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x * sigmoid(gate), [T, n] with dense rows of any stride; into ``out`` (which may be x) if given."""
+    _cuda(x, gate, out)
+    T, n = x.shape
+    _need(gate.shape == (T, n) and gate.dtype == x.dtype, "sigmoid_gate_mul: gate [T, n] of x's dtype")
+    if out is None:
+        out = torch.empty(T, n, dtype=x.dtype, device=x.device)
+    _need(out.shape == (T, n) and out.dtype == x.dtype, "sigmoid_gate_mul: out [T, n]")
+    check(_lib.mixers_lib().aphro_sigmoid_gate_mul(out.data_ptr(), _rows(out, n, "sigmoid_gate_mul out"), x.data_ptr(),
+                                                   _rows(x, n, "sigmoid_gate_mul x"), gate.data_ptr(),
+                                                   _rows(gate, n, "sigmoid_gate_mul gate"), T, n, _dt(x), _stream()), "sigmoid_gate_mul")
+    return out
+
+
+def experts_route_grouped(router_out: torch.Tensor, top: int, groups: int, keep: int, scale: float, group_top: int = 2):
+    """router_out fp32 [T, experts] -> (ids int32 [T, top], weights fp32 [T, top]): sigmoid scores, choice limited to the ``keep``
+    best of ``groups`` equal groups of neighbouring experts (a group's score: the sum of its ``group_top`` largest scores),
+    weights = score * scale."""
+    _cuda(router_out)
+    T, E = router_out.shape
+    _need(router_out.dtype == torch.float32 and router_out.is_contiguous(), "experts_route_grouped: router outputs fp32, contiguous")
+    ids = torch.empty(T, top, dtype=torch.int32, device=router_out.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=router_out.device)
+    check(_lib.mixers_lib().aphro_experts_route_grouped(ids.data_ptr(), w.data_ptr(), router_out.data_ptr(), T, E, int(top), int(groups),
+                                                        int(keep), int(group_top), float(scale), _stream()), "experts_route_grouped")
+    return ids, w

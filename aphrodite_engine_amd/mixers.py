@@ -13,7 +13,14 @@ portions and decoded tokens in one launch -- through the kernels of ``mixer_ops`
                           several maps per head over shared values, joined differentially (a_1 - lambda a_2), unit RMS per
                           head, elementwise sigmoid gate; may read another layer's keys and values instead of its own
   PolyNormMLP             down(a N(z) + b N(z^2) + c N(z^3) + e), z = up(x), N = division by the row's root mean square
-  RoutedExperts           softmax router with a choice correction, clamped gated experts, identity experts, gated shared expert
+  RoutedExperts           softmax router with a choice correction (or a sigmoid router whose choice is limited to the best groups
+                          of neighbouring experts), clamped or plain gated experts, identity experts, gated shared expert
+  HashedPairEmbedding     token embedding plus a row of a second table picked by a hash of (previous token, token); the previous
+                          token of every live request in a per-request slot
+  RotaryFrequencies       rotation frequencies with YaRN's blend of interpolated and original frequencies and its magnitude factor
+  LatentAttention         softmax attention through a low-rank latent: a token caches one row [normed latent | one rotated key part
+                          shared by all heads]; queries go through a latent of their own; elementwise sigmoid output gate
+  ClampedGLUMLP           down(g * sigmoid(alpha g) * (u + 1)) with g and u clamped, biased projections
 """
 import math
 from dataclasses import dataclass
@@ -48,6 +55,24 @@ class ConvStateSpec:
 
     def allocate(self, num_blocks: int, block_size: int, num_slots: int, dtype, device):
         return torch.zeros(num_slots, max(self.taps - 1, 0), self.channels, dtype=dtype, device=device)
+
+
+@dataclass(frozen=True)
+class LatentCacheSpec:
+    """A paged cache of one row per token that all heads share: [blocks, block, rank + rot_dim]."""
+    rank: int
+    rot_dim: int
+
+    def allocate(self, num_blocks: int, block_size: int, num_slots: int, dtype, device):
+        return torch.zeros(num_blocks, block_size, self.rank + self.rot_dim, dtype=dtype, device=device)
+
+
+@dataclass(frozen=True)
+class TokenStateSpec:
+    """The last token of every live request, one int32 per request slot."""
+
+    def allocate(self, num_blocks: int, block_size: int, num_slots: int, dtype, device):
+        return torch.zeros(num_slots, dtype=torch.int32, device=device)
 
 
 @dataclass(frozen=True)
@@ -241,15 +266,27 @@ class RoutedExperts(nn.Module):
     shared expert runs for every token, times sigmoid of a one-row product.  The router runs in fp32."""
 
     def __init__(self, width: int, ff: int, experts: int, top: int, identity: int, limit: float, dtype, shared_ff: int = 0,
-                 shared_limit: float = 0.0, alpha: float = 1.702, prefix: str = ""):
+                 shared_limit: float = 0.0, alpha: float = 1.702, prefix: str = "", score: str = "softmax", groups: int = 1,
+                 keep: int = 1, group_top: int = 2, route_scale: float = 1.0):
+        """``limit`` <= 0: experts of the plain gated form gate * sigmoid(alpha gate) * up (alpha 1: silu).  ``score``
+        "sigmoid_grouped": scores are sigmoid(router output); the experts form ``groups`` equal groups of neighbours, a group's
+        score is the sum of its ``group_top`` largest scores, only experts of the ``keep`` best groups can be chosen; the
+        weights are the chosen scores times ``route_scale``."""
         super().__init__()
         from .model import QuantLinear
         self.width, self.ff, self.experts, self.top, self.identity = width, ff, experts, top, identity
         self.limit, self.alpha, self.shared_ff, self.shared_limit = float(limit), float(alpha), shared_ff, float(shared_limit)
+        self.score, self.groups, self.keep, self.group_top, self.route_scale = score, int(groups), int(keep), int(group_top), float(route_scale)
         if not 0 < top <= experts + identity:
             raise ValueError(f"top {top} of {experts} + {identity} experts")
+        if score not in ("softmax", "sigmoid_grouped"):
+            raise ValueError(f"router score {score!r}")
+        if score == "sigmoid_grouped":
+            if identity or groups < 1 or experts % groups or not 0 < keep <= groups or top > keep * (experts // groups):
+                raise ValueError(f"{experts} experts in {groups} groups of which {keep} are kept, top {top}")
         self.router = nn.Parameter(torch.zeros(experts + identity, width, dtype=torch.float32), requires_grad=False)
-        self.correction = nn.Parameter(torch.zeros(experts + identity, dtype=torch.float32), requires_grad=False)
+        self.correction = nn.Parameter(torch.zeros(experts + identity, dtype=torch.float32), requires_grad=False) \
+            if score == "softmax" else None
         self.w_gate_up = nn.Parameter(torch.zeros(experts, 2 * ff, width, dtype=dtype), requires_grad=False)
         self.w_down = nn.Parameter(torch.zeros(experts, width, ff, dtype=dtype), requires_grad=False)
         if shared_ff:
@@ -261,10 +298,140 @@ class RoutedExperts(nn.Module):
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         z = torch.nn.functional.linear(h.float(), self.router)
-        ids, w = mops.experts_route(z, self.correction, self.top)
+        if self.score == "sigmoid_grouped":
+            ids, w = mops.experts_route_grouped(z, self.top, self.groups, self.keep, self.route_scale, self.group_top)
+        else:
+            ids, w = mops.experts_route(z, self.correction, self.top)
         shared = gate = None
         if self.shared_ff:
             s_in = self.shared_in(h)
             shared = self.shared_down(mops.clamped_glu(s_in, self.shared_ff, self.shared_limit, self.alpha))
             gate = s_in[:, 2 * self.shared_ff:2 * self.shared_ff + 1]
         return mops.experts_forward(h, ids, w, self.w_gate_up, self.w_down, self.limit, self.alpha, shared, gate)
+
+
+class HashedPairEmbedding(nn.Module):
+    """x = table[token] + pair_table[(previous * mul_prev + token * mul_cur) mod buckets]; a sequence's first token takes the
+    table's last row (number ``buckets``).  The previous token is state: one int32 per request slot (``state_spec``), read for
+    the first row of a segment that continues a sequence and advanced to the segment's last token."""
+
+    def __init__(self, vocab: int, width: int, buckets: int, mul_prev: int, mul_cur: int, dtype):
+        super().__init__()
+        if buckets < 1:
+            raise ValueError("a hashed pair table needs at least one bucket")
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        self.table = nn.Parameter(torch.empty(vocab, width, dtype=dtype), requires_grad=False)
+        self.pair_table = nn.Parameter(torch.empty(buckets + 1, width, dtype=dtype), requires_grad=False)
+
+    def state_spec(self) -> TokenStateSpec:
+        return TokenStateSpec()
+
+    def forward(self, batch: StepBatch, token_state: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return mops.hashed_pair_embed(self.table, self.pair_table, batch.input_ids, token_state, batch.state_slots, batch.q_start,
+                                      batch.q_len, batch.ctx_len, batch.seq_of_token, self.mul_prev, self.mul_cur, out=out)
+
+
+class RotaryFrequencies:
+    """Frequencies f_i = base^(-2 i / dims), i < dims / 2, of a rotation that pairs number i with number i + dims / 2, and the
+    factor on cos and sin.  With YaRN scaling (factor, original length, fast and slow turn counts): a linear ramp over i between
+    the numbers that turn ``fast`` and ``slow`` times over the original length blends f_i / factor (ramp 1) with f_i (ramp 0),
+    and cos and sin are multiplied by 0.1 ln(factor) + 1."""
+
+    def __init__(self, dims: int, base: float, factor: Optional[float] = None, original: Optional[float] = None,
+                 fast: Optional[float] = None, slow: Optional[float] = None):
+        if dims < 0 or dims % 2:
+            raise ValueError(f"{dims} rotated numbers: pairs are needed")
+        self.dims = int(dims)
+        half = dims // 2
+        f = [float(base) ** (-2.0 * i / dims) for i in range(half)]
+        self.mscale = 1.0
+        if factor is not None:
+            def number_turning(turns: float) -> float:
+                return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+            lo = max(math.floor(number_turning(fast)), 0)
+            hi = min(math.ceil(number_turning(slow)), dims - 1)
+            for i in range(half):
+                ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+                f[i] = f[i] / factor * ramp + f[i] * (1.0 - ramp)
+            self.mscale = 0.1 * math.log(factor) + 1.0
+        self.inv_freq = torch.tensor(f, dtype=torch.float32)
+
+    def to(self, device) -> "RotaryFrequencies":
+        self.inv_freq = self.inv_freq.to(device)
+        return self
+
+
+class LatentAttention(nn.Module):
+    """Causal softmax attention whose keys and values are products of a cached low-rank latent.
+
+      c_q = norm(W_dq h), q = W_uq c_q = per head [q_n (dim) | q_r (rot_dim)];   W_dkv h = [c (kv_rank) | k_r (rot_dim)], c normed
+      key of head a = [W_uk,a c | rot(k_r)], value = W_uv,a c;  score = (q_n . W_uk,a c + rot(q_r) . rot(k_r)) * scale
+      out = W_o (heads * sigmoid(W_g h))
+
+    Every projection that reads h -- W_dq, W_dkv, W_g -- is one product.  The attention itself runs in the latent (the cache
+    holds [c | rot(k_r)] per token and nothing per head): q_lat,a = W_uk,a^T q_n,a is a batched product over heads, the kernel
+    returns sum_j p_ij c_j per head, and W_uv,a is applied to that, again batched over heads."""
+
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, q_rank: int, kv_rank: int, scale: float,
+                 rotary: RotaryFrequencies, eps: float, dtype, prefix: str = ""):
+        super().__init__()
+        from .loader import merged_plan
+        from .model import QuantLinear
+        if rotary.dims > rot_dim:
+            raise ValueError(f"{rotary.dims} rotated numbers in a rotary part of {rot_dim}")
+        self.heads, self.dim, self.rot_dim, self.vdim, self.q_rank, self.kv_rank = heads, dim, rot_dim, vdim, q_rank, kv_rank
+        self.scale, self.eps, self.rotary = float(scale), float(eps), rotary
+        self.names = ["dq", "dkv", "g"]
+        self.splits = [q_rank, kv_rank + rot_dim, heads * vdim]
+        pad = -sum(self.splits) % 8               # rows of the fused product stay 16-byte multiples
+        if pad:
+            self.splits.append(pad)
+        self.in_proj = QuantLinear(width, self.splits, None, dtype, prefix=prefix + "in_proj", plan=merged_plan(self.splits))
+        self.in_proj.weight.data.zero_()
+        self.q_norm = nn.Parameter(torch.ones(q_rank, dtype=dtype), requires_grad=False)
+        self.kv_norm = nn.Parameter(torch.ones(kv_rank, dtype=dtype), requires_grad=False)
+        self.uq = QuantLinear(q_rank, [heads * (dim + rot_dim)], None, dtype, prefix=prefix + "uq")
+        self.w_uk = nn.Parameter(torch.zeros(heads, dim, kv_rank, dtype=dtype), requires_grad=False)      # rows of W_uk, head by head
+        self.w_uv = nn.Parameter(torch.zeros(heads, vdim, kv_rank, dtype=dtype), requires_grad=False)
+        self.out_proj = QuantLinear(heads * vdim, [width], None, dtype, prefix=prefix + "out_proj")
+
+    def cache_spec(self) -> LatentCacheSpec:
+        return LatentCacheSpec(self.kv_rank, self.rot_dim)
+
+    def finalize(self) -> None:
+        self.rotary.to(self.w_uk.device)
+
+    def forward(self, h: torch.Tensor, cache: torch.Tensor, batch: StepBatch) -> torch.Tensor:
+        T, H, d, P, e, R = h.shape[0], self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
+        rot = self.rotary
+        proj = self.in_proj(h)
+        cq = mops.latent_prep(proj, 0, self.q_rank, self.q_rank, R, P, rot.dims, self.q_norm, self.kv_norm, cache,
+                              batch.slot_mapping, batch.q_start, batch.ctx_len, batch.seq_of_token, rot.inv_freq, rot.mscale, self.eps)
+        q = self.uq(cq).view(T, H, d + P)
+        q_lat = torch.empty(T, H, R, dtype=h.dtype, device=h.device)
+        torch.bmm(q[:, :, :d].transpose(0, 1), self.w_uk, out=q_lat.transpose(0, 1))
+        o_lat = torch.empty(T, H, R, dtype=h.dtype, device=h.device)
+        mops.latent_attention(o_lat, q_lat, q[:, :, d:] if P else None, cache, batch.block_tables, batch.q_start, batch.q_len,
+                              batch.ctx_len, batch.seq_of_token, (min(batch.q_lens), max(batch.q_lens)), rot.inv_freq, rot.mscale,
+                              rot.dims, self.scale, max_kv_len=max(c + n for c, n in zip(batch.ctx_lens, batch.q_lens)))
+        o = torch.empty(T, H, e, dtype=h.dtype, device=h.device)
+        torch.bmm(o_lat.transpose(0, 1), self.w_uv.transpose(1, 2), out=o.transpose(0, 1))
+        o = o.view(T, H * e)
+        g_at = self.q_rank + R + P
+        mops.sigmoid_gate_mul(o, proj[:, g_at:g_at + H * e], out=o)
+        return self.out_proj(o)
+
+
+class ClampedGLUMLP(nn.Module):
+    """down(g * sigmoid(alpha g) * (u + 1)), g = min(gate h, limit), u = clamp(up h, +-limit); gate and up are one product;
+    every projection may carry a bias."""
+
+    def __init__(self, width: int, ff: int, limit: float, dtype, alpha: float = 1.702, bias: bool = True, prefix: str = ""):
+        super().__init__()
+        from .model import QuantLinear
+        self.ff, self.limit, self.alpha = ff, float(limit), float(alpha)
+        self.gate_up = QuantLinear(width, [ff, ff], None, dtype, prefix=prefix + "gate_up", bias=bias)
+        self.down = QuantLinear(ff, [width], None, dtype, prefix=prefix + "down", bias=bias)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return self.down(mops.clamped_glu(self.gate_up(h), self.ff, self.limit, self.alpha))

@@ -56,7 +56,12 @@ def _register_builtin() -> None:
         from .gipozen import load_gipozen
         return load_gipozen(model_dir, config, **kw)
 
+    def fekotar(model_dir, config, **kw):
+        from .fekotar import load_fekotar
+        return load_fekotar(model_dir, config, **kw)
+
     for arch in ("LlamaForCausalLM", "MistralForCausalLM", "MixtralForCausalLM"):
         _LOADERS.setdefault(arch, llama)
     _LOADERS.setdefault("Fatudra", fatudra)
     _LOADERS.setdefault("Gipozen", gipozen)
+    _LOADERS.setdefault("Fekotar", fekotar)

@@ -196,9 +196,53 @@ int aphro_experts_down_gemm(float* expert_out, const void* y, const void* w_down
 int aphro_experts_combine(void* out, const float* expert_out, const int32_t* ids, const float* weights, const void* h,
                       int64_t h_stride, const void* shared, int64_t shared_stride, const void* shared_gate,
                       int64_t shared_gate_stride, int64_t num_tokens, int width, int top, int experts, int dtype, void* stream);
-/* out[t, j] = g * sigmoid(alpha * g) * (u + 1), g = min(in[t, j], limit), u = clamp(in[t, d + j], +-limit), j < d */
+/* out[t, j] = g * sigmoid(alpha * g) * (u + 1), g = min(in[t, j], limit), u = clamp(in[t, d + j], +-limit), j < d;
+ * limit <= 0 (here and in aphro_experts_glu_gemm): the plain gated form in[t, j] * sigmoid(alpha * in[t, j]) * in[t, d + j] */
 int aphro_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t num_tokens, int d, float limit, float alpha,
                       int dtype, void* stream);
+
+/* ---- sublayers side by side, hashed token-pair embedding, attention through a low-rank latent ------------------------------ */
+
+/* x[t] = table[ids[t]] + pair_table[row], row = (previous * mul_prev + ids[t] * mul_cur) mod buckets, or row `buckets` for a
+ * sequence's first token (pair_table has buckets + 1 rows).  The previous token of a segment's first row is
+ * token_state[state_slots[s]] (read only if ctx_len[s] > 0).  x fp32 [T, width]. */
+int aphro_hashed_pair_embed(float* x, const void* table, const void* pair_table, const int64_t* ids, const int32_t* token_state,
+                            const int32_t* state_slots, const int32_t* q_start, const int32_t* ctx_len,
+                            const int32_t* seq_of_token, int64_t num_tokens, int width, int64_t vocab, int64_t buckets,
+                            int64_t mul_prev, int64_t mul_cur, int dtype, void* stream);
+/* token_state[state_slots[s]] = the last token of segment s (after hashed_pair_embed of the same step, on the same stream) */
+int aphro_token_state_write(int32_t* token_state, const int64_t* ids, const int32_t* state_slots, const int32_t* q_start,
+                            const int32_t* q_len, int num_seqs, void* stream);
+/* x += ya + yb + bias (each optional), then out = x / rms(x) * weight (out NULL: the add alone).  x fp32 [T, width] in place;
+ * ya, yb [T, width] of `dtype` with their row strides; bias, weight [width] of `dtype`; out [T, width] contiguous. */
+int aphro_residual_add2_rms_norm(float* x, const void* ya, int64_t ya_stride, const void* yb, int64_t yb_stride, const void* bias,
+                                 const void* weight, void* out, int64_t num_tokens, int width, float eps, int dtype, void* stream);
+
+/* Per token, from the rows of one input product (proj, row stride proj_stride): cq[t] = rms_norm(proj[t, q_at : q_at + q_rank]) *
+ * wq (q_rank 0: none); cache[slot_mapping[t]] = [rms_norm(proj[t, kv_at : kv_at + kv_rank]) * wkv | rotate(next rot_dim numbers)].
+ * cache [num_cache_rows, kv_rank + rot_dim].  The rotation turns pair (i, i + rot_dims / 2) of the first rot_dims numbers by
+ * position * inv_freq[i] and scales it by mscale; inv_freq fp32 [rot_dims / 2]. */
+int aphro_latent_prep(void* cq, void* cache, int64_t num_cache_rows, const void* proj, int64_t proj_stride, int q_at, int kv_at,
+                      const void* wq, const void* wkv, const int64_t* slot_mapping, const int32_t* q_start, const int32_t* ctx_len,
+                      const int32_t* seq_of_token, const float* inv_freq, float mscale, int64_t num_tokens, int q_rank, int kv_rank,
+                      int rot_dim, int rot_dims, float eps, int dtype, void* stream);
+/* Causal softmax attention of every head over the shared latent rows cache [blocks, block, kv_rank + rot_dim]:
+ * score = ([q_lat | rotate(q_rot)] . row) * scale, out = sum p * row[:kv_rank].  q_lat / q_rot / out are addressed as
+ * base + t * stride + head * head_stride (elements); any sizes (kv_rank <= 512), fp32 math. */
+int aphro_latent_attention_plain(void* out, int64_t out_stride, int64_t out_head_stride, const void* q_lat, int64_t ql_stride,
+                                 int64_t ql_head_stride, const void* q_rot, int64_t qr_stride, int64_t qr_head_stride,
+                                 const void* cache, const int32_t* block_tables, int max_blocks, int64_t num_blocks, int block_size,
+                                 const int32_t* q_start, const int32_t* ctx_len, const int32_t* seq_of_token, const float* inv_freq,
+                                 float mscale, int64_t num_tokens, int heads, int kv_rank, int rot_dim, int rot_dims, float scale,
+                                 int dtype, void* stream);
+/* out[t, i] = x[t, i] * sigmoid(gate[t, i]), i < n (out may be x) */
+int aphro_sigmoid_gate_mul(void* out, int64_t out_stride, const void* x, int64_t x_stride, const void* gate, int64_t gate_stride,
+                           int64_t num_tokens, int n, int dtype, void* stream);
+/* Sigmoid router limited to groups: s = sigmoid(router_out) fp32 [T, experts]; the experts form `groups` equal groups of
+ * neighbours, a group's score is the sum of its group_top largest s, only the `keep` best groups' experts can be chosen; ids
+ * int32 [T, top] are the `top` largest s among them, weights fp32 [T, top] = s * scale. */
+int aphro_experts_route_grouped(int32_t* ids, float* weights, const float* router_out, int64_t num_tokens, int experts, int top,
+                                int groups, int keep, int group_top, float scale, void* stream);
 
 #ifdef __cplusplus
 }
