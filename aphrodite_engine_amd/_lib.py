@@ -197,6 +197,9 @@ MIXERS_SIGNATURES = {
     "aphro_residual_add2_rms_norm": (I, [P, P, L, P, L, P, P, P, L, I, F, I, P]),
     "aphro_latent_prep": (I, [P, P, L, P, L, I, I, P, P, P, P, P, P, P, F, L, I, I, I, I, F, I, P]),
     "aphro_latent_attention_plain": (I, [P, L, L, P, L, L, P, L, L, P, P, I, L, I, P, P, P, P, F, L, I, I, I, I, F, I, P]),
+    "aphro_latent_attention_fast_supported": (I, [I, I, I, I]),
+    "aphro_latent_attention_splits": (I, [L, I, I, I, I]),
+    "aphro_latent_attention": (I, [P, L, L, P, L, L, P, L, L, P, P, I, L, I, P, P, P, P, P, F, L, I, I, I, I, I, I, I, F, P, L, I, P]),
     "aphro_sigmoid_gate_mul": (I, [P, L, P, L, P, L, L, I, I, P]),
     "aphro_experts_route_grouped": (I, [P, P, P, L, I, I, I, I, I, F, P]),
 }

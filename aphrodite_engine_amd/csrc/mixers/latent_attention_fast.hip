@@ -1,0 +1,397 @@
+// bf16 matrix-core path of the attention through a low-rank latent (same semantics as latent_attention.hip, which stays the
+// fp32 path and the path of sizes this does not tile).
+//
+// Every head reads the SAME cache rows [c (R) | k_r (P)], as key (all R + P numbers) and as value (the first R), so the
+// query rows of a segment are flattened: row = token * heads + head.  A workgroup of four waves owns 64 consecutive rows, 16
+// per wave -- with 16 heads a wave is one token's heads, with 64 a workgroup is -- and walks the visible keys 64 at a time:
+// the tile's cache rows come in with 16-byte loads, go to LDS once row-major (chunk-swizzled: the key operand) and, their
+// first R numbers, once transposed (the value operand); the next tile's rows are fetched into registers while the current
+// tile's products run.  S^T = K Q^T on v_mfma_f32_16x16x32_bf16, so that the probabilities come out in the B-operand layout
+// of O^T = C^T P^T; mask and online softmax (base 2) are fp32 on the accumulators.  The query operand is [q_lat | rotate(q_r)]
+// padded with zeros to a multiple of 32, built once per workgroup (the rotation in fp32 at the row's position).
+//
+// Rows that see many keys while the launch has few workgroups (decoded tokens) split their key range over grid z; the
+// partial (max, sum, accumulator) triples go through a scratch tensor and la_merge_kernel joins them.
+#include "mixers_common.h"
+
+namespace aphro {
+
+struct LAParams {
+  uint16_t* out;
+  const uint16_t* q_lat;
+  const uint16_t* q_rot;
+  const uint16_t* cache;
+  const int32_t* block_tables;
+  const int32_t* q_start;
+  const int32_t* q_len;
+  const int32_t* ctx_len;
+  const float* inv_freq;
+  int64_t out_stride, out_head_stride, ql_stride, ql_head_stride, qr_stride, qr_head_stride, num_blocks;
+  int max_blocks, block_size, bs_shift, heads, nsplit;
+  float scale, mscale;
+  float* ws;          // split partials [T * heads, nsplit, 2 + R]
+};
+
+__device__ __forceinline__ int la_slot(const LAParams& p, const int32_t* bt, int key) {
+  int blk, off;
+  if (p.bs_shift >= 0) {
+    blk = bt[key >> p.bs_shift];
+    off = key & (p.block_size - 1);
+  } else {
+    blk = bt[key / p.block_size];
+    off = key % p.block_size;
+  }
+  if (blk < 0 || blk >= p.num_blocks) blk = 0;             // never read outside the pool
+  return blk * p.block_size + off;
+}
+
+constexpr int LF_BM = 64, LF_BN = 64, LF_VT = LF_BN + 4;
+
+template <int R, int P>
+struct LFGeom {
+  static constexpr int D = R + P, DP = (D + 31) / 32 * 32, NCH = DP / 8, NKS = DP / 32, NDT = R / 16;
+  static constexpr int SWZ = (NCH & -NCH) - 1;
+  static constexpr int ITEMS = LF_BN / 2 * NCH, NI = (ITEMS + 255) / 256;
+  static constexpr size_t LDS_BYTES = (size_t)(LF_BN * DP + R * LF_VT) * sizeof(uint16_t);
+};
+
+// one thread's share of a key tile: chunks (8 numbers) of two neighbouring keys, so that the transposed stores are dwords
+template <int R, int P>
+struct LFStage {
+  u16x8 a[LFGeom<R, P>::NI], b[LFGeom<R, P>::NI];
+};
+
+template <int R, int P>
+__device__ __forceinline__ void lf_load(LFStage<R, P>& st, const LAParams& p, const int32_t* bt, int t0, int t_end) {
+  typedef LFGeom<R, P> G;
+#pragma unroll
+  for (int it = 0; it < G::NI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    u16x8 va = u16x8{0, 0, 0, 0, 0, 0, 0, 0}, vb = va;
+    if (i < G::ITEMS) {
+      const int tp = i / G::NCH, ch = i % G::NCH;
+      if (8 * ch < G::D) {
+        const int k0 = t0 + 2 * tp;
+        if (k0 < t_end) va = *reinterpret_cast<const u16x8*>(p.cache + (int64_t)la_slot(p, bt, k0) * G::D + 8 * ch);
+        if (k0 + 1 < t_end) vb = *reinterpret_cast<const u16x8*>(p.cache + (int64_t)la_slot(p, bt, k0 + 1) * G::D + 8 * ch);
+      }
+    }
+    st.a[it] = va;
+    st.b[it] = vb;
+  }
+}
+
+template <int R, int P>
+__device__ __forceinline__ void lf_store(const LFStage<R, P>& st, uint16_t* k_lds, uint16_t* vt_lds) {
+  typedef LFGeom<R, P> G;
+#pragma unroll
+  for (int it = 0; it < G::NI; ++it) {
+    const int i = threadIdx.x + 256 * it;
+    if (i < G::ITEMS) {
+      const int tp = i / G::NCH, ch = i % G::NCH;
+      const int ta = 2 * tp, tb = 2 * tp + 1;
+      *reinterpret_cast<u16x8*>(&k_lds[ta * G::DP + 8 * (ch ^ (ta & G::SWZ))]) = st.a[it];
+      *reinterpret_cast<u16x8*>(&k_lds[tb * G::DP + 8 * (ch ^ (tb & G::SWZ))]) = st.b[it];
+      if (8 * ch < R) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          *reinterpret_cast<uint32_t*>(&vt_lds[(8 * ch + j) * LF_VT + 2 * tp]) = (uint32_t)st.a[it][j] | ((uint32_t)st.b[it][j] << 16);
+      }
+    }
+  }
+}
+
+template <int R, int P>
+__global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
+  typedef LFGeom<R, P> G;
+  constexpr int NH = LF_BN / 16, NPK = LF_BN / 32;
+  extern __shared__ __attribute__((aligned(16))) uint16_t la_lds[];
+  uint16_t* k_lds = la_lds;
+  uint16_t* vt_lds = la_lds + LF_BN * G::DP;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
+  const int seq = blockIdx.y, z = blockIdx.z;
+  const int len = p.q_len[seq];
+  const int H = p.heads;
+  const int nrows = len * H;
+  const int r0 = blockIdx.x * LF_BM;
+  if (r0 >= nrows) return;
+  const int ctx = p.ctx_len[seq], s0 = p.q_start[seq];
+  const int row = r0 + 16 * wave + c;
+  const bool rvalid = row < nrows;
+  const int rowc = rvalid ? row : nrows - 1;
+  const int tok = rowc / H, head = rowc - tok * H;
+  const int qpos = ctx + tok;
+  // rows of this wave span these positions
+  const int wrow_lo = min(r0 + 16 * wave, nrows - 1), wrow_hi = min(r0 + 16 * wave + 15, nrows - 1);
+  const int wpos_lo = ctx + wrow_lo / H, wpos_hi = ctx + wrow_hi / H;
+  const int nk = ctx + min(r0 + LF_BM - 1, nrows - 1) / H + 1;          // keys the workgroup's last row sees
+  // this workgroup's share of the key tiles
+  const int tiles = (nk + LF_BN - 1) / LF_BN, per = (tiles + p.nsplit - 1) / p.nsplit;
+  const int t_begin = z * per * LF_BN, t_end = min(nk, (z + 1) * per * LF_BN);
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float qs = p.scale * LOG2E;
+
+  // the query operand: [q_lat | rotate(q_rot) | zeros]
+  u32x4 qf[G::NKS];
+  {
+    const uint16_t* ql = p.q_lat + (int64_t)(s0 + tok) * p.ql_stride + (int64_t)head * p.ql_head_stride;
+    const uint16_t* qr = P ? p.q_rot + (int64_t)(s0 + tok) * p.qr_stride + (int64_t)head * p.qr_head_stride : nullptr;
+#pragma unroll
+    for (int ks = 0; ks < G::NKS; ++ks) {
+      const int at = 32 * ks + 8 * g;
+      u32x4 v = u32x4{0, 0, 0, 0};
+      if (at < R) {
+        v = *reinterpret_cast<const u32x4*>(ql + at);
+      } else if (at < G::D) {
+        constexpr int HALF = P / 2;
+        const int i0 = at - R;
+        const bool low = i0 < HALF;
+        const int f0 = low ? i0 : i0 - HALF;
+        const u16x8 mine = *reinterpret_cast<const u16x8*>(qr + i0);
+        const u16x8 other = *reinterpret_cast<const u16x8*>(qr + (low ? i0 + HALF : i0 - HALF));
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float a = (float)qpos * p.inv_freq[f0 + j];
+          const float cs = cosf(a) * p.mscale, sn = sinf(a) * p.mscale;
+          const float x = BFloat::to_f32(mine[j]), y = BFloat::to_f32(other[j]);
+          o[j] = low ? x * cs - y * sn : x * cs + y * sn;
+        }
+        v = u32x4{pack2_16<true>(o[0], o[1]), pack2_16<true>(o[2], o[3]), pack2_16<true>(o[4], o[5]), pack2_16<true>(o[6], o[7])};
+      }
+      qf[ks] = v;
+    }
+  }
+  f32x4 o[G::NDT];
+#pragma unroll
+  for (int i = 0; i < G::NDT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -1e30f, l_run = 0.f;
+  const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
+  const int kmax = min(qpos, t_end - 1);                    // the last key this row takes from this workgroup's share
+
+  LFStage<R, P> st;
+  if (t_begin < t_end) lf_load<R, P>(st, p, bt, t_begin, t_end);
+  for (int t0 = t_begin; t0 < t_end; t0 += LF_BN) {
+    __syncthreads();                                        // the previous tile is consumed
+    lf_store<R, P>(st, k_lds, vt_lds);
+    __syncthreads();
+    if (t0 + LF_BN < t_end) lf_load<R, P>(st, p, bt, t0 + LF_BN, t_end);       // in flight during this tile's products
+    if (t0 > wpos_hi) continue;                             // every key of the tile is ahead of the wave's rows
+    f32x4 s[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      s[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int tk = 16 * h + c;
+#pragma unroll
+      for (int ks = 0; ks < G::NKS; ++ks) {
+        const int ch = (4 * ks + g) ^ (tk & G::SWZ);
+        const u32x4 kf = *reinterpret_cast<const u32x4*>(&k_lds[tk * G::DP + 8 * ch]);
+        s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[h], 0, 0, 0);
+      }
+    }
+    const bool edge = t0 + LF_BN - 1 > min(wpos_lo, t_end - 1);   // some key of the tile is not for some row of the wave
+    float pv[NH][4];
+    float mx = -1e30f;
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float xv = s[h][r] * qs;
+        if (edge) xv = t0 + 16 * h + 4 * g + r <= kmax ? xv : -1e30f;
+        pv[h][r] = xv;
+        mx = fmaxf(mx, xv);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
+    float lsum = 0.f;
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float e = pv[h][r] > -1e29f ? __builtin_amdgcn_exp2f(pv[h][r] - m_new) : 0.f;
+        pv[h][r] = e;
+        lsum += e;
+      }
+    l_run = l_run * alpha + lsum;
+#pragma unroll
+    for (int dt = 0; dt < G::NDT; ++dt) o[dt] *= alpha;
+    u32x4 pf[NPK];
+#pragma unroll
+    for (int pk = 0; pk < NPK; ++pk)
+      pf[pk] = u32x4{pack2_16<true>(pv[2 * pk][0], pv[2 * pk][1]), pack2_16<true>(pv[2 * pk][2], pv[2 * pk][3]),
+                     pack2_16<true>(pv[2 * pk + 1][0], pv[2 * pk + 1][1]), pack2_16<true>(pv[2 * pk + 1][2], pv[2 * pk + 1][3])};
+#pragma unroll
+    for (int pk = 0; pk < NPK; ++pk) {
+#pragma unroll
+      for (int dt = 0; dt < G::NDT; ++dt) {
+        const uint16_t* vr = &vt_lds[(16 * dt + c) * LF_VT + 32 * pk + 4 * g];
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(vr);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(vr + 16);
+        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[pk]), o[dt], 0, 0, 0);
+      }
+    }
+  }
+  float l = l_run;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!rvalid) return;
+  if (p.nsplit == 1) {
+    const float f = l > 0.f ? 1.f / l : 0.f;
+    uint16_t* op = p.out + (int64_t)(s0 + tok) * p.out_stride + (int64_t)head * p.out_head_stride;
+#pragma unroll
+    for (int dt = 0; dt < G::NDT; ++dt)
+      *reinterpret_cast<u32x2*>(op + 16 * dt + 4 * g) = u32x2{pack2_16<true>(o[dt][0] * f, o[dt][1] * f), pack2_16<true>(o[dt][2] * f, o[dt][3] * f)};
+  } else {
+    float* wp = p.ws + (((int64_t)(s0 + tok) * H + head) * p.nsplit + z) * (2 + R);
+    if (g == 0) {
+      wp[0] = m_run;
+      wp[1] = l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < G::NDT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) wp[2 + 16 * dt + 4 * g + r] = o[dt][r];
+  }
+}
+
+// one wave per (token, head): joins the nsplit partial results
+__global__ void la_merge_kernel(uint16_t* __restrict__ out, int64_t out_stride, int64_t out_head_stride, const float* __restrict__ ws,
+                                int heads, int nsplit, int R) {
+  const int64_t t = blockIdx.x;
+  const int head = blockIdx.y;
+  const float* wp = ws + ((t * heads + head) * nsplit) * (int64_t)(2 + R);
+  float M = -1e30f;
+  for (int zz = 0; zz < nsplit; ++zz) M = fmaxf(M, wp[(int64_t)zz * (2 + R)]);
+  float L = 0.f;
+  for (int zz = 0; zz < nsplit; ++zz) L += wp[(int64_t)zz * (2 + R) + 1] * __builtin_amdgcn_exp2f(wp[(int64_t)zz * (2 + R)] - M);
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  uint16_t* op = out + t * out_stride + (int64_t)head * out_head_stride;
+  for (int col = threadIdx.x; col < R; col += blockDim.x) {
+    float acc = 0.f;
+    for (int zz = 0; zz < nsplit; ++zz) {
+      const float* w = wp + (int64_t)zz * (2 + R);
+      if (w[1] > 0.f) acc += w[2 + col] * __builtin_amdgcn_exp2f(w[0] - M);
+    }
+    op[col] = BFloat::from_f32(acc * inv);
+  }
+}
+
+template <int R, int P>
+static int la_launch(const LAParams& p, int num_seqs, int max_q_len, int64_t num_tokens, hipStream_t stream) {
+  typedef LFGeom<R, P> G;
+  static bool configured = false;
+  if (!configured) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(la_mfma_kernel<R, P>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES);
+    if (e != hipSuccess) {
+      set_error("latent_attention: %zu bytes of LDS refused: %s", G::LDS_BYTES, hipGetErrorString(e));
+      return APHRO_ERR_INVALID;
+    }
+    configured = true;
+  }
+  const int64_t tiles = ((int64_t)max_q_len * p.heads + LF_BM - 1) / LF_BM;
+  hipLaunchKernelGGL((la_mfma_kernel<R, P>), dim3((unsigned)tiles, (unsigned)num_seqs, (unsigned)p.nsplit), dim3(256), G::LDS_BYTES,
+                     stream, p);
+  if (p.nsplit > 1)
+    hipLaunchKernelGGL(la_merge_kernel, dim3((unsigned)num_tokens, (unsigned)p.heads), dim3(64), 0, stream, p.out, p.out_stride,
+                       p.out_head_stride, p.ws, p.heads, p.nsplit, R);
+  return APHRO_OK;
+}
+
+}  // namespace aphro
+
+using namespace aphro;
+
+extern "C" int aphro_latent_attention_plain(void* out, int64_t out_stride, int64_t out_head_stride, const void* q_lat,
+                                            int64_t ql_stride, int64_t ql_head_stride, const void* q_rot, int64_t qr_stride,
+                                            int64_t qr_head_stride, const void* cache, const int32_t* block_tables, int max_blocks,
+                                            int64_t num_blocks, int block_size, const int32_t* q_start, const int32_t* ctx_len,
+                                            const int32_t* seq_of_token, const float* inv_freq, float mscale, int64_t num_tokens,
+                                            int heads, int kv_rank, int rot_dim, int rot_dims, float scale, int dtype,
+                                            void* stream);
+
+#define LA_FAST_SIZES(X) X(128, 16) X(128, 32) X(256, 32) X(256, 64) X(512, 64)
+
+extern "C" int aphro_latent_attention_fast_supported(int kv_rank, int rot_dim, int rot_dims, int dtype) {
+  if (dtype != APHRO_BF16 || rot_dims != rot_dim) return 0;
+#define LA_IS(R_, P_) if (kv_rank == R_ && rot_dim == P_) return 1;
+  LA_FAST_SIZES(LA_IS)
+#undef LA_IS
+  return 0;
+}
+
+/* The number of key-range splits the matrix-core kernel would use, and so the scratch it needs: floats = num_tokens * heads *
+ * splits * (2 + kv_rank) when splits > 1. */
+extern "C" int aphro_latent_attention_splits(int64_t num_tokens, int num_seqs, int max_q_len, int heads, int max_kv_len) {
+  const int64_t tiles = ((int64_t)max_q_len * heads + LF_BM - 1) / LF_BM * num_seqs;
+  if (tiles >= 128 || max_kv_len < 512) return 1;
+  int s = max_kv_len / 256;
+  const int64_t room = 512 / (tiles > 0 ? tiles : 1);
+  if (s > room) s = (int)room;
+  if (s > 16) s = 16;
+  return s < 1 ? 1 : s;
+}
+
+extern "C" int aphro_latent_attention(void* out, int64_t out_stride, int64_t out_head_stride, const void* q_lat, int64_t ql_stride,
+                                      int64_t ql_head_stride, const void* q_rot, int64_t qr_stride, int64_t qr_head_stride,
+                                      const void* cache, const int32_t* block_tables, int max_blocks, int64_t num_blocks,
+                                      int block_size, const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
+                                      const int32_t* seq_of_token, const float* inv_freq, float mscale, int64_t num_tokens,
+                                      int num_seqs, int max_q_len, int max_kv_len, int heads, int kv_rank, int rot_dim, int rot_dims,
+                                      float scale, float* workspace, int64_t workspace_floats, int dtype, void* stream) {
+  if (num_tokens == 0) return APHRO_OK;
+  const auto al16 = [](const void* ptr) { return ((uintptr_t)ptr & 15) == 0; };
+  const bool fast = aphro_latent_attention_fast_supported(kv_rank, rot_dim, rot_dims, dtype) && q_len && num_seqs > 0 && max_q_len > 0 &&
+                    al16(q_lat) && al16(q_rot) && al16(cache) && al16(out) && ql_stride % 8 == 0 && ql_head_stride % 8 == 0 &&
+                    qr_stride % 8 == 0 && qr_head_stride % 8 == 0 && out_stride % 4 == 0 && out_head_stride % 4 == 0 &&
+                    (int64_t)max_q_len * heads < (1 << 30);
+  if (!fast)
+    return aphro_latent_attention_plain(out, out_stride, out_head_stride, q_lat, ql_stride, ql_head_stride, q_rot, qr_stride,
+                                        qr_head_stride, cache, block_tables, max_blocks, num_blocks, block_size, q_start, ctx_len,
+                                        seq_of_token, inv_freq, mscale, num_tokens, heads, kv_rank, rot_dim, rot_dims, scale, dtype,
+                                        stream);
+  APHRO_CHECK(out && q_lat && q_rot && cache && block_tables && q_start && ctx_len && inv_freq, "latent_attention: null argument");
+  APHRO_CHECK(heads > 0 && heads <= 65535 && block_size > 0 && max_blocks > 0 && num_blocks > 0 && num_seqs <= 65535,
+              "latent_attention: bad geometry");
+  LAParams p;
+  p.out = (uint16_t*)out;
+  p.q_lat = (const uint16_t*)q_lat;
+  p.q_rot = (const uint16_t*)q_rot;
+  p.cache = (const uint16_t*)cache;
+  p.block_tables = block_tables;
+  p.q_start = q_start;
+  p.q_len = q_len;
+  p.ctx_len = ctx_len;
+  p.inv_freq = inv_freq;
+  p.out_stride = out_stride;
+  p.out_head_stride = out_head_stride;
+  p.ql_stride = ql_stride;
+  p.ql_head_stride = ql_head_stride;
+  p.qr_stride = qr_stride;
+  p.qr_head_stride = qr_head_stride;
+  p.num_blocks = num_blocks;
+  p.max_blocks = max_blocks;
+  p.block_size = block_size;
+  p.bs_shift = (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
+  p.heads = heads;
+  p.scale = scale;
+  p.mscale = mscale;
+  p.nsplit = 1;
+  p.ws = nullptr;
+  const int want = aphro_latent_attention_splits(num_tokens, num_seqs, max_q_len, heads, max_kv_len);
+  if (want > 1 && workspace && workspace_floats >= num_tokens * (int64_t)heads * want * (2 + kv_rank)) {
+    p.nsplit = want;
+    p.ws = workspace;
+  }
+  int rc = APHRO_ERR_INVALID;
+#define LA_GO(R_, P_) if (kv_rank == R_ && rot_dim == P_) rc = la_launch<R_, P_>(p, num_seqs, max_q_len, num_tokens, (hipStream_t)stream);
+  LA_FAST_SIZES(LA_GO)
+#undef LA_GO
+  if (rc != APHRO_OK) return rc;
+  APHRO_LAUNCH_CHECK();
+  return APHRO_OK;
+}

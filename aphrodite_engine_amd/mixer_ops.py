@@ -582,11 +582,12 @@ def _head_view(t: torch.Tensor, T: int, heads: int, n: int, what: str):
 def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: Optional[torch.Tensor], cache: torch.Tensor,
                      block_tables: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor,
                      seq_of_token: torch.Tensor, q_len_range, inv_freq: Optional[torch.Tensor], mscale: float, rot_dims: int,
-                     scale: float, max_kv_len: int = 0) -> None:
+                     scale: float, max_kv_len: int = 0, plain: bool = False) -> None:
     """Causal softmax attention of a batch of segments over latent cache rows [c | k_r] that all heads share.  q_lat
     [T, heads, kv_rank] (every head's query carried into the latent), q_rot [T, heads, rot_dim] (raw: rotated here at the row's
     position), out [T, heads, kv_rank] = sum_j p_ij c_j -- any strides over tokens and heads.  ``q_len_range`` (shortest, longest
-    segment) and ``max_kv_len`` (longest ctx_len + q_len), known on the host, choose the kernel and its work split."""
+    segment) and ``max_kv_len`` (longest ctx_len + q_len), known on the host, choose the work split of the matrix-core kernel,
+    which serves the sizes ``latent_attention_fast_supported`` names; ``plain`` forces the fp32-math kernel of any size."""
     _cuda(out, q_lat, q_rot, cache, block_tables, q_start, q_len, ctx_len, seq_of_token, inv_freq)
     T, H, R = q_lat.shape
     nb, bs, D = cache.shape
@@ -606,10 +607,30 @@ def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: Optional[tor
     _i32(seq_of_token, T, "seq_of_token")
     _need(rot_dims == 0 or (inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2
                             and inv_freq.is_contiguous()), "latent_attention: inv_freq fp32 [rot_dims / 2]")
-    check(_lib.mixers_lib().aphro_latent_attention_plain(
+    lib = _lib.mixers_lib()
+    if plain:
+        check(lib.aphro_latent_attention_plain(
+            out.data_ptr(), os_, ohs, q_lat.data_ptr(), qs, qhs, _p(q_rot), rs, rhs, cache.data_ptr(), block_tables.data_ptr(),
+            block_tables.shape[1], nb, bs, q_start.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), _p(inv_freq), float(mscale),
+            T, H, R, P_, int(rot_dims), float(scale), _dt(q_lat), _stream()), "latent_attention")
+        return
+    lo, hi = int(q_len_range[0]), int(q_len_range[1])
+    _need(0 < lo <= hi, "latent_attention: q_len_range (shortest, longest)")
+    ws, ws_n = None, 0
+    if lib.aphro_latent_attention_fast_supported(R, P_, int(rot_dims), _dt(q_lat)):
+        splits = int(lib.aphro_latent_attention_splits(T, S, hi, H, int(max_kv_len)))
+        if splits > 1:
+            ws_n = T * H * splits * (2 + R)
+            ws = torch.empty(ws_n, dtype=torch.float32, device=q_lat.device)
+    check(lib.aphro_latent_attention(
         out.data_ptr(), os_, ohs, q_lat.data_ptr(), qs, qhs, _p(q_rot), rs, rhs, cache.data_ptr(), block_tables.data_ptr(),
-        block_tables.shape[1], nb, bs, q_start.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), _p(inv_freq), float(mscale), T,
-        H, R, P_, int(rot_dims), float(scale), _dt(q_lat), _stream()), "latent_attention")
+        block_tables.shape[1], nb, bs, q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), _p(inv_freq),
+        float(mscale), T, S, hi, int(max_kv_len), H, R, P_, int(rot_dims), float(scale), _p(ws), ws_n, _dt(q_lat), _stream()),
+        "latent_attention")
+
+
+def latent_attention_fast_supported(kv_rank: int, rot_dim: int, rot_dims: int, dtype: torch.dtype) -> bool:
+    return dtype in _DT and bool(_lib.mixers_lib().aphro_latent_attention_fast_supported(kv_rank, rot_dim, rot_dims, _DT[dtype]))
 
 
 def sigmoid_gate_mul(x: torch.Tensor, gate: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -235,6 +235,20 @@ int aphro_latent_attention_plain(void* out, int64_t out_stride, int64_t out_head
                                  const int32_t* q_start, const int32_t* ctx_len, const int32_t* seq_of_token, const float* inv_freq,
                                  float mscale, int64_t num_tokens, int heads, int kv_rank, int rot_dim, int rot_dims, float scale,
                                  int dtype, void* stream);
+/* The same attention with the kernel chosen by size: bf16 with (kv_rank, rot_dim) in {(128, 16), (128, 32), (256, 32), (256, 64),
+ * (512, 64)}, rot_dims == rot_dim and 16-byte aligned rows run on the matrix cores (aphro_latent_attention_fast_supported), the
+ * query rows of a segment flattened to (token, head) pairs, 64 per workgroup; everything else runs the kernel above.  min/max
+ * segment lengths and the longest ctx_len + q_len come from the host.  Decode-sized launches split long key ranges over
+ * aphro_latent_attention_splits(...) workgroups when `workspace` holds num_tokens * heads * splits * (2 + kv_rank) floats. */
+int aphro_latent_attention_fast_supported(int kv_rank, int rot_dim, int rot_dims, int dtype);
+int aphro_latent_attention_splits(int64_t num_tokens, int num_seqs, int max_q_len, int heads, int max_kv_len);
+int aphro_latent_attention(void* out, int64_t out_stride, int64_t out_head_stride, const void* q_lat, int64_t ql_stride,
+                           int64_t ql_head_stride, const void* q_rot, int64_t qr_stride, int64_t qr_head_stride, const void* cache,
+                           const int32_t* block_tables, int max_blocks, int64_t num_blocks, int block_size, const int32_t* q_start,
+                           const int32_t* q_len, const int32_t* ctx_len, const int32_t* seq_of_token, const float* inv_freq,
+                           float mscale, int64_t num_tokens, int num_seqs, int max_q_len, int max_kv_len, int heads, int kv_rank,
+                           int rot_dim, int rot_dims, float scale, float* workspace, int64_t workspace_floats, int dtype,
+                           void* stream);
 /* out[t, i] = x[t, i] * sigmoid(gate[t, i]), i < n (out may be x) */
 int aphro_sigmoid_gate_mul(void* out, int64_t out_stride, const void* x, int64_t x_stride, const void* gate, int64_t gate_stride,
                            int64_t num_tokens, int n, int dtype, void* stream);
