@@ -1,10 +1,15 @@
-"""``bench.py --mixers [--mixers-design fatudra|gipozen]``: prefill and decode throughput of a Fatudra (or Gipozen) stack at sizes that resemble a real model's layers
+"""``bench.py --mixers [--mixers-design fatudra|gipozen|fekotar]``: prefill and decode throughput of a Fatudra (or Gipozen) stack at sizes that resemble a real model's layers
 (random bf16 weights), beside a Llama stack of equal width / heads / feed-forward / layer count on the unquantised op path,
 plus each mixer kernel alone against its roofline and against the like kernel of the Llama path.  Prints ONE JSON line;
 the default workload of bench.py is untouched by it.  The Gipozen stack: windowed differential attention (two maps of half the
 head size over shared values, window 1024 + 4 kept tokens, 4-tap convolutions), every second layer reading the previous
 layer's keys and values and carrying 16 + 1 experts (top 4, a quarter of the dense feed-forward each, one shared expert)
 instead of the PolyNorm feed-forward; its expert products are priced against the MFMA figure over the ACTIVE experts' flops.
+
+The Fekotar stack: attention through a cached latent of rank 512 + 64 rotated numbers (queries through a latent of 3/8 of the
+width), heads of 128 + 64 / 128, a dense clamped feed-forward in the first layer and 16 silu experts (top 4 of the 2 best of 4
+groups, a quarter of the dense feed-forward each) in the others; it stands beside Llama AND beside the Gipozen stack (the
+closest existing model: its own attention kernels plus routed experts) at equal width.
 
 Rooflines used: 8 TB/s HBM for the memory-bound kernels (norms, activations, decode attention, the decode step of the
 memories: their state is read and written once), 2.5 PFLOP/s dense bf16 MFMA for prompt attention (4 d flops per visible
@@ -59,6 +64,22 @@ def gipozen_config(s):
 
 
 GIP_WINDOW, GIP_KEEP, GIP_EXPERTS, GIP_TOP = 1024, 4, 16, 4
+
+
+FEK_RANK, FEK_ROT, FEK_EXPERTS, FEK_TOP, FEK_GROUPS, FEK_KEEP = 512, 64, 16, 4, 4, 2
+
+
+def fekotar_config(s):
+    mixer = {"heads": s["heads"], "dim": s["dim"], "rot_dim": FEK_ROT, "vdim": s["dim"], "q_rank": s["width"] * 3 // 8, "kv_rank": FEK_RANK,
+             "scale": (s["dim"] + FEK_ROT) ** -0.5,
+             "rot": {"base": 10000.0, "dims": FEK_ROT, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    eff = s["ff"] // 4 // 32 * 32
+    dense = {"kind": "dense", "ff": s["ff"], "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": eff},
+           "router": {"experts": FEK_EXPERTS, "top": FEK_TOP, "scale": 1.0, "groups": {"count": FEK_GROUPS, "keep": FEK_KEEP}}}
+    layers = [{"type": "latent_attention", "mixer": dict(mixer), "mlp": dense if i == 0 else moe} for i in range(LAYERS)]
+    return {"architecture": "Fekotar", "vocab": VOCAB, "width": s["width"], "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": layers}
 
 
 def timed(fn, iters=10, warmup=3):
@@ -313,10 +334,129 @@ def gipozen_kernel_section(s, prompt_len, batch, ctx, device):
     return out
 
 
+def fekotar_kernel_section(s, prompt_len, batch, ctx, device):
+    """Each Fekotar kernel alone at the stack's shapes, and the like kernel of the Llama path at the same shapes."""
+    from . import _custom_ops as ops
+    from . import mixer_ops as mops
+    from .mixers import LatentCacheSpec, RotaryFrequencies
+    bf = torch.bfloat16
+    H, G, d, W, ff = s["heads"], s["kv_heads"], s["dim"], s["width"], s["ff"]
+    R, P, Rq = FEK_RANK, FEK_ROT, s["width"] * 3 // 8
+    eff = ff // 4 // 32 * 32
+    pre, dec, pages = batches(prompt_len, batch, ctx, device, VOCAB)
+    out = {}
+
+    def rec(name, sec, bytes_=None, flops=None, like=None):
+        r = {"us": round(sec * 1e6, 1)}
+        if bytes_ is not None:
+            r["frac_hbm"] = round(bytes_ / sec / HBM, 3)
+        if flops is not None:
+            r["frac_mfma"] = round(flops / sec / MFMA, 4)
+        if like is not None:
+            r["like"] = like
+        out[name] = r
+
+    rot = RotaryFrequencies(P, 10000.0, 4.0, 4096, 32.0, 1.0).to(device)
+    cache = LatentCacheSpec(R, P).allocate(pages, BLOCK, batch, bf, device)
+    cache.normal_()
+    for name, b, T in (("prefill", pre, prompt_len), ("decode", dec, batch)):
+        # ---- attention in the latent: every head over the shared rows -----------------------------------------------------------
+        q_lat = torch.randn(T, H, R, device=device, dtype=bf) * R ** -0.5
+        q = torch.randn(T, H, d + P, device=device, dtype=bf)
+        o = torch.empty(T, H, R, device=device, dtype=bf)
+        sec = timed(lambda: mops.latent_attention(o, q_lat, q[:, :, d:], cache, b.block_tables, b.q_start, b.q_len, b.ctx_len,
+                                                  b.seq_of_token, (min(b.q_lens), max(b.q_lens)), rot.inv_freq, rot.mscale, P,
+                                                  (d + P) ** -0.5, max_kv_len=max(c + n for c, n in zip(b.ctx_lens, b.q_lens))))
+        lq = torch.randn(T, H, d, device=device, dtype=bf)
+        if name == "prefill":
+            pairs = T * (T + 1) / 2
+            flops = pairs * H * (2.0 * (R + P) + 2.0 * R)
+            k = torch.randn(T, G, d, device=device, dtype=bf)
+            v = torch.randn(T, G, d, device=device, dtype=bf)
+            cu = torch.tensor([0, T], dtype=torch.int32, device=device)
+            lsec = timed(lambda: ops.flash_attn_varlen(lq, k, v, cu, T, d ** -0.5, causal=True))
+            rec("attention_prefill", sec, flops=flops, like={"kernel": "flash_attn_varlen", "us": round(lsec * 1e6, 1),
+                                                             "frac_mfma": round(pairs * H * 4.0 * d / lsec / MFMA, 4)})
+        else:
+            nbytes = batch * (ctx + 1) * (R + P) * 2
+            lk = torch.randn(pages, G, d // 8, BLOCK, 8, device=device, dtype=bf)
+            lv = torch.randn(pages, G, d, BLOCK, device=device, dtype=bf)
+            lens = torch.full((batch, ), ctx + 1, dtype=torch.int32, device=device)
+            lo = torch.empty(T, H, d, device=device, dtype=bf)
+            lsec = timed(lambda: ops.paged_attention_v1(lo, lq, lk, lv, G, d ** -0.5, b.block_tables, lens, BLOCK, ctx + 1, None,
+                                                        "auto", 1.0, 1.0))
+            lbytes = batch * (ctx + 1) * G * 2 * d * 2
+            rec("attention_decode", sec, bytes_=nbytes, like={"kernel": "paged_attention_v1", "us": round(lsec * 1e6, 1),
+                                                              "frac_hbm": round(lbytes / lsec / HBM, 3)})
+        # ---- norms of the latents + rotation + cache write -----------------------------------------------------------------------
+        proj = torch.randn(T, Rq + R + P + H * d, device=device, dtype=bf)
+        wq, wkv = torch.randn(Rq, device=device, dtype=bf), torch.randn(R, device=device, dtype=bf)
+        sec = timed(lambda: mops.latent_prep(proj, 0, Rq, Rq, R, P, P, wq, wkv, cache, b.slot_mapping, b.q_start, b.ctx_len,
+                                             b.seq_of_token, rot.inv_freq, rot.mscale, 1e-6))
+        k = torch.randn(T, G, d, device=device, dtype=bf)
+        lkc = torch.zeros(pages, G, d // 8, BLOCK, 8, device=device, dtype=bf)
+        lvc = torch.zeros(pages, G, d, BLOCK, device=device, dtype=bf)
+        lqq = torch.randn(T, H * d, device=device, dtype=bf)
+        lkk = torch.randn(T, G * d, device=device, dtype=bf)
+        cs = torch.randn(8192, d, device=device, dtype=bf)
+        lsec = timed(lambda: (ops.rotary_embedding(b.positions, lqq, lkk, d, cs, True),
+                              ops.reshape_and_cache(k, k, lkc, lvc, b.slot_mapping, "auto", 1.0, 1.0)))
+        rec("latent_prep_" + name, sec, bytes_=T * (Rq + R + P) * 4,
+            like={"kernel": "rotary_embedding + reshape_and_cache", "us": round(lsec * 1e6, 1),
+                  "frac_hbm": round(T * (H + 3 * G) * d * 4 / lsec / HBM, 3)})
+        # ---- output gate, both sublayers' residual add + norm, the dense activation, the embedding ----------------------------------
+        og, gg = torch.randn(T, H * d, device=device, dtype=bf), torch.randn(T, H * d, device=device, dtype=bf)
+        sec = timed(lambda: mops.sigmoid_gate_mul(og, gg, out=og))
+        rec("sigmoid_gate_mul_" + name, sec, bytes_=T * H * d * 6)
+        x = torch.randn(T, W, device=device)
+        ya, yb = torch.randn(T, W, device=device, dtype=bf), torch.randn(T, W, device=device, dtype=bf)
+        w16 = torch.randn(W, device=device, dtype=bf)
+        sec = timed(lambda: mops.residual_add2_rms_norm(x, ya, yb, weight=w16))
+        x16, r16 = torch.randn(T, W, device=device, dtype=bf), torch.randn(T, W, device=device, dtype=bf)
+        lsec = timed(lambda: ops.fused_add_rms_norm(x16, r16, w16, 1e-5))
+        rec("residual_add2_rms_norm_" + name, sec, bytes_=T * W * (4 + 4 + 2 + 2 + 2),
+            like={"kernel": "fused_add_rms_norm", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * W * 8 / lsec / HBM, 3)})
+        gu = torch.randn(T, 2 * ff, device=device, dtype=bf)
+        sec = timed(lambda: mops.clamped_glu(gu, ff, 7.0, 1.702))
+        lo2 = torch.empty(T, ff, device=device, dtype=bf)
+        lsec = timed(lambda: ops.silu_and_mul(lo2, gu))
+        rec("clamped_glu_" + name, sec, bytes_=T * ff * 6,
+            like={"kernel": "silu_and_mul", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * ff * 6 / lsec / HBM, 3)})
+        table, pair = torch.randn(VOCAB, W, device=device, dtype=bf), torch.randn(65522, W, device=device, dtype=bf)
+        tstate = torch.zeros(batch, dtype=torch.int32, device=device)
+        sec = timed(lambda: mops.hashed_pair_embed(table, pair, b.input_ids, tstate, b.state_slots, b.q_start, b.q_len, b.ctx_len,
+                                                   b.seq_of_token, 31, 7))
+        rec("hashed_pair_embed_" + name, sec, bytes_=T * W * 8)
+        # ---- experts: route, sort, both products, combine -- against the dense feed-forward's library products of equal active size
+        h = torch.randn(T, W, device=device, dtype=bf)
+        zr = torch.randn(T, FEK_EXPERTS, device=device)
+        ids, wts = mops.experts_route_grouped(zr, FEK_TOP, FEK_GROUPS, FEK_KEEP, 1.0)
+        wgu = torch.randn(FEK_EXPERTS, 2 * eff, W, device=device, dtype=bf) * W ** -0.5
+        wdn = torch.randn(FEK_EXPERTS, W, eff, device=device, dtype=bf) * eff ** -0.5
+        sec = timed(lambda: mops.experts_forward(h, ids, wts, wgu, wdn, 0.0, 1.0))
+        wl1 = torch.randn(2 * FEK_TOP * eff, W, device=device, dtype=bf)
+        wl2 = torch.randn(W, FEK_TOP * eff, device=device, dtype=bf)
+        act = torch.randn(T, FEK_TOP * eff, device=device, dtype=bf)
+        lsec = timed(lambda: (torch.nn.functional.linear(h, wl1), torch.nn.functional.linear(act, wl2)))
+        flops = 6.0 * T * FEK_TOP * eff * W
+        r = {"kernel": "library products of the dense feed-forward at the active size", "us": round(lsec * 1e6, 1)}
+        if name == "prefill":
+            r["frac_mfma"] = round(flops / lsec / MFMA, 4)
+            rec("experts_" + name, sec, flops=flops, like=r)
+        else:
+            r["frac_hbm"] = round(3 * FEK_TOP * eff * W * 2 / lsec / HBM, 3)
+            rec("experts_" + name, sec, bytes_=FEK_EXPERTS * 3 * eff * W * 2, like=r)
+        sec = timed(lambda: mops.experts_route_grouped(zr, FEK_TOP, FEK_GROUPS, FEK_KEEP, 1.0))
+        rec("experts_route_grouped_" + name, sec)
+    return out
+
+
 def main(args) -> int:
     from . import _lib
     if getattr(args, "mixers_design", "fatudra") == "gipozen":
         return main_gipozen(args)
+    if getattr(args, "mixers_design", "fatudra") == "fekotar":
+        return main_fekotar(args)
     from .fatudra import FatudraConfig, FatudraForCausalLM
     from .model import LlamaConfig, LlamaForCausalLM
     _lib.lib()
@@ -376,6 +516,44 @@ def main_gipozen(args) -> int:
             r["llama"] = model_throughput(llama, prompt_len, batch, ctx, device, VOCAB)
             del llama
             r["kernels"] = gipozen_kernel_section(s, prompt_len, batch, ctx, device)
+            r["seconds"] = round(time.time() - t0, 1)
+            result["sizes"][name] = r
+            torch.cuda.empty_cache()
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+def main_fekotar(args) -> int:
+    from . import _lib
+    from .fekotar import FekotarConfig, FekotarForCausalLM
+    from .gipozen import GipozenConfig, GipozenForCausalLM
+    from .model import LlamaConfig, LlamaForCausalLM
+    _lib.lib()
+    _lib.mixers_lib()
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    prompt_len, batch, ctx = args.mixers_prompt, args.batch, args.ctx
+    result = {"metric": "fekotar_vs_llama_bf16_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+              "n_gpus": 1, "layers": LAYERS, "sizes": {}}
+    with torch.no_grad():
+        for name, s in SIZES.items():
+            if args.mixers_size and name != args.mixers_size:
+                continue
+            t0 = time.time()
+            fek = FekotarForCausalLM(FekotarConfig.from_dict(fekotar_config(s)), torch.bfloat16).init_synthetic(device)
+            r = {"fekotar": model_throughput(fek, prompt_len, batch, ctx, device, VOCAB)}
+            del fek
+            gip = GipozenForCausalLM(GipozenConfig.from_dict(gipozen_config(s)), torch.bfloat16).init_synthetic(device)
+            r["gipozen"] = model_throughput(gip, prompt_len, batch, ctx, device, VOCAB)
+            del gip
+            lc = LlamaConfig(hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=LAYERS,
+                             num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], vocab_size=VOCAB,
+                             max_position_embeddings=max(8192, prompt_len + 16))
+            llama = LlamaForCausalLM(lc, None, torch.bfloat16).init_synthetic(device)
+            llama.use_fused_decode = False
+            r["llama"] = model_throughput(llama, prompt_len, batch, ctx, device, VOCAB)
+            del llama
+            r["kernels"] = fekotar_kernel_section(s, prompt_len, batch, ctx, device)
             r["seconds"] = round(time.time() - t0, 1)
             result["sizes"][name] = r
             torch.cuda.empty_cache()
