@@ -5,7 +5,8 @@
 // query rows of a segment are flattened: row = token * heads + head.  A workgroup of four waves owns 64 consecutive rows, 16
 // per wave -- with 16 heads a wave is one token's heads, with 64 a workgroup is -- and walks the visible keys 64 at a time:
 // the tile's cache rows come in with 16-byte loads, go to LDS once row-major (chunk-swizzled: the key operand) and, their
-// first R numbers, once transposed (the value operand); the next tile's rows are fetched into registers while the current
+// first R numbers, once transposed (the value operand; a layout both its stores and its reads pass without bank conflicts beyond
+// the unavoidable); the next tile's rows are fetched into registers while the current
 // tile's products run.  S^T = K Q^T on v_mfma_f32_16x16x32_bf16, so that the probabilities come out in the B-operand layout
 // of O^T = C^T P^T; mask and online softmax (base 2) are fp32 on the accumulators.  The query operand is [q_lat | rotate(q_r)]
 // padded with zeros to a multiple of 32, built once per workgroup (the rotation in fp32 at the row's position).
@@ -45,17 +46,24 @@ __device__ __forceinline__ int la_slot(const LAParams& p, const int32_t* bt, int
   return blk * p.block_size + off;
 }
 
-constexpr int LF_BM = 64, LF_BN = 64, LF_VT = LF_BN + 4;
+constexpr int LF_BM = 64, LF_BN = 64;
+// A thread brings in 16-byte chunks c8, c8 + 8, ... of ONE pair of neighbouring keys (pair = tid / 8, c8 = tid % 8): eight lanes
+// fetch a whole 128-byte line, and a tile costs a thread two block-table lookups.
+// The transposed copy of a tile: column col of the latent is a row of LF_VS dwords (64 keys and padding) at row number
+// (col & 7) * JS + (col >> 3), LF_VS = 8 mod 32 and JS = 1 mod 4.  A store instruction writes one dword per lane for 8 chunks x 8
+// key pairs -- 8 c8 + pair: two lanes per bank, the minimum -- and the value-operand reads of 16 columns x 4 key groups x 2
+// dwords land on every bank equally often.
+constexpr int LF_VS = 40;
 
 template <int R, int P>
 struct LFGeom {
   static constexpr int D = R + P, DP = (D + 31) / 32 * 32, NCH = DP / 8, NKS = DP / 32, NDT = R / 16;
-  static constexpr int SWZ = (NCH & -NCH) - 1;
-  static constexpr int ITEMS = LF_BN / 2 * NCH, NI = (ITEMS + 255) / 256;
-  static constexpr size_t LDS_BYTES = (size_t)(LF_BN * DP + R * LF_VT) * sizeof(uint16_t);
+  static constexpr int SWZ = ((NCH & -NCH) - 1) & 7;       // chunk index ^ (key & SWZ): fragment reads spread over the banks
+  static constexpr int NI = (NCH + 7) / 8;
+  static constexpr int JS = (R / 8) | 1;
+  static constexpr size_t LDS_BYTES = (size_t)LF_BN * DP * sizeof(uint16_t) + (size_t)8 * JS * LF_VS * sizeof(uint32_t);
 };
 
-// one thread's share of a key tile: chunks (8 numbers) of two neighbouring keys, so that the transposed stores are dwords
 template <int R, int P>
 struct LFStage {
   u16x8 a[LFGeom<R, P>::NI], b[LFGeom<R, P>::NI];
@@ -64,17 +72,17 @@ struct LFStage {
 template <int R, int P>
 __device__ __forceinline__ void lf_load(LFStage<R, P>& st, const LAParams& p, const int32_t* bt, int t0, int t_end) {
   typedef LFGeom<R, P> G;
+  const int tp = threadIdx.x >> 3, c8 = threadIdx.x & 7;
+  const int k0 = t0 + 2 * tp;
+  const bool ina = k0 < t_end, inb = k0 + 1 < t_end;
+  const uint16_t* ra = p.cache + (int64_t)la_slot(p, bt, ina ? k0 : t0) * G::D + 8 * c8;
+  const uint16_t* rb = p.cache + (int64_t)la_slot(p, bt, inb ? k0 + 1 : t0) * G::D + 8 * c8;
 #pragma unroll
   for (int it = 0; it < G::NI; ++it) {
-    const int i = threadIdx.x + 256 * it;
     u16x8 va = u16x8{0, 0, 0, 0, 0, 0, 0, 0}, vb = va;
-    if (i < G::ITEMS) {
-      const int tp = i / G::NCH, ch = i % G::NCH;
-      if (8 * ch < G::D) {
-        const int k0 = t0 + 2 * tp;
-        if (k0 < t_end) va = *reinterpret_cast<const u16x8*>(p.cache + (int64_t)la_slot(p, bt, k0) * G::D + 8 * ch);
-        if (k0 + 1 < t_end) vb = *reinterpret_cast<const u16x8*>(p.cache + (int64_t)la_slot(p, bt, k0 + 1) * G::D + 8 * ch);
-      }
+    if (64 * it + 8 * c8 < G::D) {
+      if (ina) va = *reinterpret_cast<const u16x8*>(ra + 64 * it);
+      if (inb) vb = *reinterpret_cast<const u16x8*>(rb + 64 * it);
     }
     st.a[it] = va;
     st.b[it] = vb;
@@ -82,20 +90,25 @@ __device__ __forceinline__ void lf_load(LFStage<R, P>& st, const LAParams& p, co
 }
 
 template <int R, int P>
-__device__ __forceinline__ void lf_store(const LFStage<R, P>& st, uint16_t* k_lds, uint16_t* vt_lds) {
+__device__ __forceinline__ void lf_store(const LFStage<R, P>& st, uint16_t* k_lds, uint32_t* vt_lds) {
   typedef LFGeom<R, P> G;
+  const int tp = threadIdx.x >> 3, c8 = threadIdx.x & 7;
+  const int ta = 2 * tp, tb = 2 * tp + 1;
+  uint16_t* ka = k_lds + ta * G::DP + 8 * (c8 ^ (ta & G::SWZ));      // chunk c8 + 8 it: the swizzle stays within the low 3 bits
+  uint16_t* kb = k_lds + tb * G::DP + 8 * (c8 ^ (tb & G::SWZ));
+  uint32_t* vt = vt_lds + c8 * LF_VS + tp;
 #pragma unroll
   for (int it = 0; it < G::NI; ++it) {
-    const int i = threadIdx.x + 256 * it;
-    if (i < G::ITEMS) {
-      const int tp = i / G::NCH, ch = i % G::NCH;
-      const int ta = 2 * tp, tb = 2 * tp + 1;
-      *reinterpret_cast<u16x8*>(&k_lds[ta * G::DP + 8 * (ch ^ (ta & G::SWZ))]) = st.a[it];
-      *reinterpret_cast<u16x8*>(&k_lds[tb * G::DP + 8 * (ch ^ (tb & G::SWZ))]) = st.b[it];
-      if (8 * ch < R) {
+    if (8 * it + c8 < G::NCH) {
+      *reinterpret_cast<u16x8*>(ka + 64 * it) = st.a[it];
+      *reinterpret_cast<u16x8*>(kb + 64 * it) = st.b[it];
+    }
+    if (64 * it + 8 * c8 < R) {
+      const u32x4 wa = __builtin_bit_cast(u32x4, st.a[it]), wb = __builtin_bit_cast(u32x4, st.b[it]);
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          *reinterpret_cast<uint32_t*>(&vt_lds[(8 * ch + j) * LF_VT + 2 * tp]) = (uint32_t)st.a[it][j] | ((uint32_t)st.b[it][j] << 16);
+      for (int j2 = 0; j2 < 4; ++j2) {        // numbers 2 j2 and 2 j2 + 1 of both keys: low halves, then high halves
+        vt[((2 * j2) * G::JS + 8 * it) * LF_VS] = __builtin_amdgcn_perm(wb[j2], wa[j2], 0x05040100);
+        vt[((2 * j2 + 1) * G::JS + 8 * it) * LF_VS] = __builtin_amdgcn_perm(wb[j2], wa[j2], 0x07060302);
       }
     }
   }
@@ -107,7 +120,7 @@ __global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
   constexpr int NH = LF_BN / 16, NPK = LF_BN / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t la_lds[];
   uint16_t* k_lds = la_lds;
-  uint16_t* vt_lds = la_lds + LF_BN * G::DP;
+  uint32_t* vt_lds = reinterpret_cast<uint32_t*>(la_lds + LF_BN * G::DP);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
   const int seq = blockIdx.y, z = blockIdx.z;
   const int len = p.q_len[seq];
@@ -169,6 +182,10 @@ __global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
   const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
   const int kmax = min(qpos, t_end - 1);                    // the last key this row takes from this workgroup's share
 
+  const uint16_t* krow[2] = {k_lds + c * G::DP + 8 * (g ^ (c & G::SWZ)), k_lds + c * G::DP + 8 * ((4 | g) ^ (c & G::SWZ))};
+  const uint32_t* vrow = vt_lds + ((c & 7) * G::JS + (c >> 3)) * LF_VS + 2 * g;
+  const bool idle = r0 + 16 * wave >= nrows;                // a wave without rows only helps to move the tiles
+
   LFStage<R, P> st;
   if (t_begin < t_end) lf_load<R, P>(st, p, bt, t_begin, t_end);
   for (int t0 = t_begin; t0 < t_end; t0 += LF_BN) {
@@ -176,16 +193,15 @@ __global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
     lf_store<R, P>(st, k_lds, vt_lds);
     __syncthreads();
     if (t0 + LF_BN < t_end) lf_load<R, P>(st, p, bt, t0 + LF_BN, t_end);       // in flight during this tile's products
-    if (t0 > wpos_hi) continue;                             // every key of the tile is ahead of the wave's rows
+    if (idle || t0 > wpos_hi) continue;                     // every key of the tile is ahead of the wave's rows
     f32x4 s[NH];
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
       s[h] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const int tk = 16 * h + c;
 #pragma unroll
       for (int ks = 0; ks < G::NKS; ++ks) {
-        const int ch = (4 * ks + g) ^ (tk & G::SWZ);
-        const u32x4 kf = *reinterpret_cast<const u32x4*>(&k_lds[tk * G::DP + 8 * ch]);
+        // chunk (4 ks + g) ^ (key & SWZ) = 8 (ks / 2) + (((ks & 1) * 4 + g) ^ (c & SWZ)): two lane offsets, the rest is immediate
+        const u32x4 kf = *reinterpret_cast<const u32x4*>(krow[ks & 1] + (16 * h) * G::DP + 64 * (ks >> 1));
         s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[h], 0, 0, 0);
       }
     }
@@ -227,10 +243,8 @@ __global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
     for (int pk = 0; pk < NPK; ++pk) {
 #pragma unroll
       for (int dt = 0; dt < G::NDT; ++dt) {
-        const uint16_t* vr = &vt_lds[(16 * dt + c) * LF_VT + 32 * pk + 4 * g];
-        const u32x2 lo = *reinterpret_cast<const u32x2*>(vr);
-        const u32x2 hi = *reinterpret_cast<const u32x2*>(vr + 16);
-        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+        const uint32_t* vr = vrow + 2 * dt * LF_VS + 16 * pk;
+        const u32x4 vf = {vr[0], vr[1], vr[8], vr[9]};
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[pk]), o[dt], 0, 0, 0);
       }
     }
@@ -330,7 +344,7 @@ extern "C" int aphro_latent_attention_splits(int64_t num_tokens, int num_seqs, i
   const int64_t tiles = ((int64_t)max_q_len * heads + LF_BM - 1) / LF_BM * num_seqs;
   if (tiles >= 128 || max_kv_len < 512) return 1;
   int s = max_kv_len / 256;
-  const int64_t room = 512 / (tiles > 0 ? tiles : 1);
+  const int64_t room = 256 / (tiles > 0 ? tiles : 1);
   if (s > room) s = (int)room;
   if (s > 16) s = 16;
   return s < 1 ? 1 : s;
