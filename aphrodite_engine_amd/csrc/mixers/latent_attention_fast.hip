@@ -2,8 +2,10 @@
 // fp32 path and the path of sizes this does not tile).
 //
 // Every head reads the SAME cache rows [c (R) | k_r (P)], as key (all R + P numbers) and as value (the first R), so the
-// query rows of a segment are flattened: row = token * heads + head.  A workgroup of four waves owns 64 consecutive rows, 16
-// per wave -- with 16 heads a wave is one token's heads, with 64 a workgroup is -- and walks the visible keys 64 at a time:
+// query rows of a segment are flattened: row = token * heads + head.  A workgroup of eight waves owns 64 consecutive rows: a
+// PAIR of waves shares 16 rows -- with 16 heads that is one token's heads -- both compute the rows' scores, each accumulates
+// one half of the R output columns (two waves per SIMD hide each other's LDS latency, and half the accumulators leave
+// registers for fragments in flight).  The workgroup walks the visible keys 64 at a time:
 // the tile's cache rows come in with 16-byte loads, go to LDS once row-major (chunk-swizzled: the key operand) and, their
 // first R numbers, once transposed (the value operand; a layout both its stores and its reads pass without bank conflicts beyond
 // the unavoidable); the next tile's rows are fetched into registers while the current
@@ -47,19 +49,19 @@ __device__ __forceinline__ int la_slot(const LAParams& p, const int32_t* bt, int
 }
 
 constexpr int LF_BM = 64, LF_BN = 64;
-// A thread brings in 16-byte chunks c8, c8 + 8, ... of ONE pair of neighbouring keys (pair = tid / 8, c8 = tid % 8): eight lanes
-// fetch a whole 128-byte line, and a tile costs a thread two block-table lookups.
+// A thread brings in 16-byte chunks cl, cl + 16, ... of ONE pair of neighbouring keys (pair = tid / 16, cl = tid % 16): sixteen
+// lanes fetch 256 contiguous bytes, and a tile costs a thread two block-table lookups.
 // The transposed copy of a tile: column col of the latent is a row of LF_VS dwords (64 keys and padding) at row number
-// (col & 7) * JS + (col >> 3), LF_VS = 8 mod 32 and JS = 1 mod 4.  A store instruction writes one dword per lane for 8 chunks x 8
-// key pairs -- 8 c8 + pair: two lanes per bank, the minimum -- and the value-operand reads of 16 columns x 4 key groups x 2
+// (col & 7) * JS + (col >> 3), LF_VS = 4 mod 32 and JS odd.  A store instruction writes one dword per lane for 16 chunks x 4
+// key pairs -- 4 cl + pair: two lanes per bank, the minimum -- and the value-operand reads of 16 columns x 4 key groups x 2
 // dwords land on every bank equally often.
-constexpr int LF_VS = 40;
+constexpr int LF_VS = 36, LF_THREADS = 512, LF_CL = 16;
 
 template <int R, int P>
 struct LFGeom {
   static constexpr int D = R + P, DP = (D + 31) / 32 * 32, NCH = DP / 8, NKS = DP / 32, NDT = R / 16;
   static constexpr int SWZ = ((NCH & -NCH) - 1) & 7;       // chunk index ^ (key & SWZ): fragment reads spread over the banks
-  static constexpr int NI = (NCH + 7) / 8;
+  static constexpr int NI = (NCH + LF_CL - 1) / LF_CL, NDH = NDT / 2;
   static constexpr int JS = (R / 8) | 1;
   static constexpr size_t LDS_BYTES = (size_t)LF_BN * DP * sizeof(uint16_t) + (size_t)8 * JS * LF_VS * sizeof(uint32_t);
 };
@@ -72,7 +74,7 @@ struct LFStage {
 template <int R, int P>
 __device__ __forceinline__ void lf_load(LFStage<R, P>& st, const LAParams& p, const int32_t* bt, int t0, int t_end) {
   typedef LFGeom<R, P> G;
-  const int tp = threadIdx.x >> 3, c8 = threadIdx.x & 7;
+  const int tp = threadIdx.x / LF_CL, c8 = threadIdx.x % LF_CL;
   const int k0 = t0 + 2 * tp;
   const bool ina = k0 < t_end, inb = k0 + 1 < t_end;
   const uint16_t* ra = p.cache + (int64_t)la_slot(p, bt, ina ? k0 : t0) * G::D + 8 * c8;
@@ -80,9 +82,9 @@ __device__ __forceinline__ void lf_load(LFStage<R, P>& st, const LAParams& p, co
 #pragma unroll
   for (int it = 0; it < G::NI; ++it) {
     u16x8 va = u16x8{0, 0, 0, 0, 0, 0, 0, 0}, vb = va;
-    if (64 * it + 8 * c8 < G::D) {
-      if (ina) va = *reinterpret_cast<const u16x8*>(ra + 64 * it);
-      if (inb) vb = *reinterpret_cast<const u16x8*>(rb + 64 * it);
+    if (8 * LF_CL * it + 8 * c8 < G::D) {
+      if (ina) va = *reinterpret_cast<const u16x8*>(ra + 8 * LF_CL * it);
+      if (inb) vb = *reinterpret_cast<const u16x8*>(rb + 8 * LF_CL * it);
     }
     st.a[it] = va;
     st.b[it] = vb;
@@ -92,36 +94,37 @@ __device__ __forceinline__ void lf_load(LFStage<R, P>& st, const LAParams& p, co
 template <int R, int P>
 __device__ __forceinline__ void lf_store(const LFStage<R, P>& st, uint16_t* k_lds, uint32_t* vt_lds) {
   typedef LFGeom<R, P> G;
-  const int tp = threadIdx.x >> 3, c8 = threadIdx.x & 7;
+  const int tp = threadIdx.x / LF_CL, c8 = threadIdx.x % LF_CL;
   const int ta = 2 * tp, tb = 2 * tp + 1;
-  uint16_t* ka = k_lds + ta * G::DP + 8 * (c8 ^ (ta & G::SWZ));      // chunk c8 + 8 it: the swizzle stays within the low 3 bits
+  uint16_t* ka = k_lds + ta * G::DP + 8 * (c8 ^ (ta & G::SWZ));      // chunk c8 + 16 it: the swizzle stays within the low 3 bits
   uint16_t* kb = k_lds + tb * G::DP + 8 * (c8 ^ (tb & G::SWZ));
   uint32_t* vt = vt_lds + c8 * LF_VS + tp;
 #pragma unroll
   for (int it = 0; it < G::NI; ++it) {
-    if (8 * it + c8 < G::NCH) {
-      *reinterpret_cast<u16x8*>(ka + 64 * it) = st.a[it];
-      *reinterpret_cast<u16x8*>(kb + 64 * it) = st.b[it];
+    if (LF_CL * it + c8 < G::NCH) {
+      *reinterpret_cast<u16x8*>(ka + 8 * LF_CL * it) = st.a[it];
+      *reinterpret_cast<u16x8*>(kb + 8 * LF_CL * it) = st.b[it];
     }
-    if (64 * it + 8 * c8 < R) {
+    if (8 * LF_CL * it + 8 * c8 < R) {
       const u32x4 wa = __builtin_bit_cast(u32x4, st.a[it]), wb = __builtin_bit_cast(u32x4, st.b[it]);
 #pragma unroll
       for (int j2 = 0; j2 < 4; ++j2) {        // numbers 2 j2 and 2 j2 + 1 of both keys: low halves, then high halves
-        vt[((2 * j2) * G::JS + 8 * it) * LF_VS] = __builtin_amdgcn_perm(wb[j2], wa[j2], 0x05040100);
-        vt[((2 * j2 + 1) * G::JS + 8 * it) * LF_VS] = __builtin_amdgcn_perm(wb[j2], wa[j2], 0x07060302);
+        vt[((2 * j2) * G::JS + LF_CL * it) * LF_VS] = __builtin_amdgcn_perm(wb[j2], wa[j2], 0x05040100);
+        vt[((2 * j2 + 1) * G::JS + LF_CL * it) * LF_VS] = __builtin_amdgcn_perm(wb[j2], wa[j2], 0x07060302);
       }
     }
   }
 }
 
 template <int R, int P>
-__global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
+__global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   typedef LFGeom<R, P> G;
   constexpr int NH = LF_BN / 16, NPK = LF_BN / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t la_lds[];
   uint16_t* k_lds = la_lds;
   uint32_t* vt_lds = reinterpret_cast<uint32_t*>(la_lds + LF_BN * G::DP);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
+  // waves 2 k and 2 k + 1 share row group k: a launch with one row group (decoded tokens of 16 heads) still uses two SIMDs
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 7, half = (threadIdx.x >> 6) & 1, g = lane >> 4, c = lane & 15;
   const int seq = blockIdx.y, z = blockIdx.z;
   const int len = p.q_len[seq];
   const int H = p.heads;
@@ -175,15 +178,15 @@ __global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
       qf[ks] = v;
     }
   }
-  f32x4 o[G::NDT];
+  f32x4 o[G::NDH];                                          // this wave's half of the output columns
 #pragma unroll
-  for (int i = 0; i < G::NDT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < G::NDH; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -1e30f, l_run = 0.f;
   const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
   const int kmax = min(qpos, t_end - 1);                    // the last key this row takes from this workgroup's share
 
   const uint16_t* krow[2] = {k_lds + c * G::DP + 8 * (g ^ (c & G::SWZ)), k_lds + c * G::DP + 8 * ((4 | g) ^ (c & G::SWZ))};
-  const uint32_t* vrow = vt_lds + ((c & 7) * G::JS + (c >> 3)) * LF_VS + 2 * g;
+  const uint32_t* vrow = vt_lds + ((c & 7) * G::JS + (c >> 3) + 2 * G::NDH * half) * LF_VS + 2 * g;
   const bool idle = r0 + 16 * wave >= nrows;                // a wave without rows only helps to move the tiles
 
   LFStage<R, P> st;
@@ -233,7 +236,7 @@ __global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
       }
     l_run = l_run * alpha + lsum;
 #pragma unroll
-    for (int dt = 0; dt < G::NDT; ++dt) o[dt] *= alpha;
+    for (int dt = 0; dt < G::NDH; ++dt) o[dt] *= alpha;
     u32x4 pf[NPK];
 #pragma unroll
     for (int pk = 0; pk < NPK; ++pk)
@@ -242,7 +245,7 @@ __global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
 #pragma unroll
     for (int pk = 0; pk < NPK; ++pk) {
 #pragma unroll
-      for (int dt = 0; dt < G::NDT; ++dt) {
+      for (int dt = 0; dt < G::NDH; ++dt) {
         const uint32_t* vr = vrow + 2 * dt * LF_VS + 16 * pk;
         const u32x4 vf = {vr[0], vr[1], vr[8], vr[9]};
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[pk]), o[dt], 0, 0, 0);
@@ -255,43 +258,55 @@ __global__ __launch_bounds__(256) void la_mfma_kernel(LAParams p) {
   if (!rvalid) return;
   if (p.nsplit == 1) {
     const float f = l > 0.f ? 1.f / l : 0.f;
-    uint16_t* op = p.out + (int64_t)(s0 + tok) * p.out_stride + (int64_t)head * p.out_head_stride;
+    uint16_t* op = p.out + (int64_t)(s0 + tok) * p.out_stride + (int64_t)head * p.out_head_stride + 16 * G::NDH * half;
 #pragma unroll
-    for (int dt = 0; dt < G::NDT; ++dt)
+    for (int dt = 0; dt < G::NDH; ++dt)
       *reinterpret_cast<u32x2*>(op + 16 * dt + 4 * g) = u32x2{pack2_16<true>(o[dt][0] * f, o[dt][1] * f), pack2_16<true>(o[dt][2] * f, o[dt][3] * f)};
   } else {
     float* wp = p.ws + (((int64_t)(s0 + tok) * H + head) * p.nsplit + z) * (2 + R);
-    if (g == 0) {
+    if (g == 0 && half == 0) {
       wp[0] = m_run;
       wp[1] = l;
     }
 #pragma unroll
-    for (int dt = 0; dt < G::NDT; ++dt)
+    for (int dt = 0; dt < G::NDH; ++dt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) wp[2 + 16 * dt + 4 * g + r] = o[dt][r];
+      for (int r = 0; r < 4; ++r) wp[2 + 16 * (G::NDH * half + dt) + 4 * g + r] = o[dt][r];
   }
 }
 
-// one wave per (token, head): joins the nsplit partial results
+// one workgroup per (token, head): joins the nsplit partial results; a thread owns two neighbouring columns and has every
+// split's piece in flight before it adds them up
+constexpr int LA_MAX_SPLIT = 16;
 __global__ void la_merge_kernel(uint16_t* __restrict__ out, int64_t out_stride, int64_t out_head_stride, const float* __restrict__ ws,
                                 int heads, int nsplit, int R) {
   const int64_t t = blockIdx.x;
   const int head = blockIdx.y;
   const float* wp = ws + ((t * heads + head) * nsplit) * (int64_t)(2 + R);
-  float M = -1e30f;
-  for (int zz = 0; zz < nsplit; ++zz) M = fmaxf(M, wp[(int64_t)zz * (2 + R)]);
-  float L = 0.f;
-  for (int zz = 0; zz < nsplit; ++zz) L += wp[(int64_t)zz * (2 + R) + 1] * __builtin_amdgcn_exp2f(wp[(int64_t)zz * (2 + R)] - M);
-  const float inv = L > 0.f ? 1.f / L : 0.f;
-  uint16_t* op = out + t * out_stride + (int64_t)head * out_head_stride;
-  for (int col = threadIdx.x; col < R; col += blockDim.x) {
-    float acc = 0.f;
-    for (int zz = 0; zz < nsplit; ++zz) {
-      const float* w = wp + (int64_t)zz * (2 + R);
-      if (w[1] > 0.f) acc += w[2 + col] * __builtin_amdgcn_exp2f(w[0] - M);
+  const int col = 2 * threadIdx.x;
+  f32x2 ml[LA_MAX_SPLIT], v[LA_MAX_SPLIT];
+#pragma unroll
+  for (int zz = 0; zz < LA_MAX_SPLIT; ++zz)
+    if (zz < nsplit) {
+      ml[zz] = *reinterpret_cast<const f32x2*>(wp + (int64_t)zz * (2 + R));
+      v[zz] = col < R ? *reinterpret_cast<const f32x2*>(wp + (int64_t)zz * (2 + R) + 2 + col) : f32x2{0.f, 0.f};
     }
-    op[col] = BFloat::from_f32(acc * inv);
-  }
+  float M = -1e30f;
+#pragma unroll
+  for (int zz = 0; zz < LA_MAX_SPLIT; ++zz)
+    if (zz < nsplit) M = fmaxf(M, ml[zz][0]);
+  float L = 0.f, a0 = 0.f, a1 = 0.f;
+#pragma unroll
+  for (int zz = 0; zz < LA_MAX_SPLIT; ++zz)
+    if (zz < nsplit && ml[zz][1] > 0.f) {
+      const float f = __builtin_amdgcn_exp2f(ml[zz][0] - M);
+      L += ml[zz][1] * f;
+      a0 += v[zz][0] * f;
+      a1 += v[zz][1] * f;
+    }
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  if (col < R)
+    *reinterpret_cast<uint32_t*>(out + t * out_stride + (int64_t)head * out_head_stride + col) = pack2_16<true>(a0 * inv, a1 * inv);
 }
 
 template <int R, int P>
@@ -308,11 +323,11 @@ static int la_launch(const LAParams& p, int num_seqs, int max_q_len, int64_t num
     configured = true;
   }
   const int64_t tiles = ((int64_t)max_q_len * p.heads + LF_BM - 1) / LF_BM;
-  hipLaunchKernelGGL((la_mfma_kernel<R, P>), dim3((unsigned)tiles, (unsigned)num_seqs, (unsigned)p.nsplit), dim3(256), G::LDS_BYTES,
+  hipLaunchKernelGGL((la_mfma_kernel<R, P>), dim3((unsigned)tiles, (unsigned)num_seqs, (unsigned)p.nsplit), dim3(LF_THREADS), G::LDS_BYTES,
                      stream, p);
   if (p.nsplit > 1)
-    hipLaunchKernelGGL(la_merge_kernel, dim3((unsigned)num_tokens, (unsigned)p.heads), dim3(64), 0, stream, p.out, p.out_stride,
-                       p.out_head_stride, p.ws, p.heads, p.nsplit, R);
+    hipLaunchKernelGGL(la_merge_kernel, dim3((unsigned)num_tokens, (unsigned)p.heads), dim3((R / 2 + 63) / 64 * 64), 0, stream, p.out,
+                       p.out_stride, p.out_head_stride, p.ws, p.heads, p.nsplit, R);
   return APHRO_OK;
 }
 
@@ -343,10 +358,10 @@ extern "C" int aphro_latent_attention_fast_supported(int kv_rank, int rot_dim, i
 extern "C" int aphro_latent_attention_splits(int64_t num_tokens, int num_seqs, int max_q_len, int heads, int max_kv_len) {
   const int64_t tiles = ((int64_t)max_q_len * heads + LF_BM - 1) / LF_BM * num_seqs;
   if (tiles >= 128 || max_kv_len < 512) return 1;
-  int s = max_kv_len / 256;
-  const int64_t room = 256 / (tiles > 0 ? tiles : 1);
+  int s = max_kv_len / 128;                                // two tiles of keys per workgroup
+  const int64_t room = 512 / (tiles > 0 ? tiles : 1);
   if (s > room) s = (int)room;
-  if (s > 16) s = 16;
+  if (s > LA_MAX_SPLIT) s = LA_MAX_SPLIT;
   return s < 1 ? 1 : s;
 }
 
