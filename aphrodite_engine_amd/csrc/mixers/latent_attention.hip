@@ -32,24 +32,23 @@ __global__ void latent_prep_kernel(typename T::storage* __restrict__ cq, typenam
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
   const typename T::storage* row = proj + t * proj_stride;
+  float ssq = 0.f, ss = 0.f;                                  // both statistics are gathered before either is waited for
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) {
+    const float v = T::to_f32(row[q_at + i]);
+    ssq += v * v;
+  }
+  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) {
+    const float v = T::to_f32(row[kv_at + i]);
+    ss += v * v;
+  }
   if (q_rank > 0) {
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < q_rank; i += blockDim.x) {
-      const float v = T::to_f32(row[q_at + i]);
-      ss += v * v;
-    }
-    const float rstd = 1.0f / sqrtf(wg_sum(ss, red) / (float)q_rank + eps);
+    const float rstd = 1.0f / sqrtf(wg_sum(ssq, red) / (float)q_rank + eps);
     for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
       cq[t * (int64_t)q_rank + i] = T::from_f32(T::to_f32(row[q_at + i]) * rstd * T::to_f32(wq[i]));
   }
   const int64_t slot = slot_mapping[t];
   if (slot < 0 || slot >= num_cache_rows) return;             // a padded row
   typename T::storage* dst = cache + slot * (int64_t)(kv_rank + rot_dim);
-  float ss = 0.f;
-  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) {
-    const float v = T::to_f32(row[kv_at + i]);
-    ss += v * v;
-  }
   const float rstd = 1.0f / sqrtf(wg_sum(ss, red) / (float)kv_rank + eps);
   for (int i = threadIdx.x; i < kv_rank; i += blockDim.x)
     dst[i] = T::from_f32(T::to_f32(row[kv_at + i]) * rstd * T::to_f32(wkv[i]));
@@ -205,6 +204,32 @@ __global__ void sigmoid_gate_mul_kernel(typename T::storage* __restrict__ out, i
   out[t * out_stride + i] = T::from_f32(T::to_f32(x[t * x_stride + i]) * sigmoid_f(T::to_f32(gate[t * gate_stride + i])));
 }
 
+template <typename T>
+__global__ void sigmoid_gate_mul_vec8_kernel(typename T::storage* __restrict__ out, int64_t out_stride,
+                                             const typename T::storage* __restrict__ x, int64_t x_stride,
+                                             const typename T::storage* __restrict__ gate, int64_t gate_stride, int n) {
+  const int64_t t = blockIdx.x;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (i >= n) return;
+  if constexpr (sizeof(typename T::storage) == 2) {
+    const u16x8 xv = *reinterpret_cast<const u16x8*>(x + t * x_stride + i), gv = *reinterpret_cast<const u16x8*>(gate + t * gate_stride + i);
+    u16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = T::from_f32(T::to_f32(xv[j]) * sigmoid_f(T::to_f32(gv[j])));
+    *reinterpret_cast<u16x8*>(out + t * out_stride + i) = r;
+  } else {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const f32x4 xv = *reinterpret_cast<const f32x4*>(x + t * x_stride + i + 4 * h);
+      const f32x4 gv = *reinterpret_cast<const f32x4*>(gate + t * gate_stride + i + 4 * h);
+      f32x4 r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = xv[j] * sigmoid_f(gv[j]);
+      *reinterpret_cast<f32x4*>(out + t * out_stride + i + 4 * h) = r;
+    }
+  }
+}
+
 }  // namespace aphro
 
 using namespace aphro;
@@ -277,10 +302,16 @@ extern "C" int aphro_sigmoid_gate_mul(void* out, int64_t out_stride, const void*
   if (num_tokens == 0) return APHRO_OK;
   APHRO_CHECK(out && x && gate && n > 0 && out_stride >= n && x_stride >= n && gate_stride >= n && (n + 255) / 256 <= 65535,
               "sigmoid_gate_mul: bad arguments");
+  const auto al16 = [](const void* ptr) { return ((uintptr_t)ptr & 15) == 0; };
+  const bool vec = n % 8 == 0 && out_stride % 8 == 0 && x_stride % 8 == 0 && gate_stride % 8 == 0 && al16(out) && al16(x) && al16(gate);
   MIX_DISPATCH_DTYPE(dtype, {
     typedef typename T::storage S;
-    hipLaunchKernelGGL((sigmoid_gate_mul_kernel<T>), dim3((unsigned)num_tokens, (unsigned)((n + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, (S*)out, out_stride, (const S*)x, x_stride, (const S*)gate, gate_stride, n);
+    if (vec)
+      hipLaunchKernelGGL((sigmoid_gate_mul_vec8_kernel<T>), dim3((unsigned)num_tokens, (unsigned)((n / 8 + 255) / 256)), dim3(256), 0,
+                         (hipStream_t)stream, (S*)out, out_stride, (const S*)x, x_stride, (const S*)gate, gate_stride, n);
+    else
+      hipLaunchKernelGGL((sigmoid_gate_mul_kernel<T>), dim3((unsigned)num_tokens, (unsigned)((n + 255) / 256)), dim3(256), 0,
+                         (hipStream_t)stream, (S*)out, out_stride, (const S*)x, x_stride, (const S*)gate, gate_stride, n);
   });
   APHRO_LAUNCH_CHECK();
   return APHRO_OK;

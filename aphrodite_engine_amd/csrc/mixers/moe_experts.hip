@@ -515,6 +515,38 @@ __global__ void clamped_glu_kernel(typename T::storage* __restrict__ out, const 
   out[t * (int64_t)d + i] = T::from_f32(clamped_glu_f(T::to_f32(in[t * in_stride + i]), T::to_f32(in[t * in_stride + d + i]), limit, alpha));
 }
 
+// 8 neighbouring elements per thread where the rows allow 16-byte accesses
+template <typename T>
+__global__ void clamped_glu_vec8_kernel(typename T::storage* __restrict__ out, const typename T::storage* __restrict__ in,
+                                        int64_t in_stride, int d, float limit, float alpha) {
+  const int64_t t = blockIdx.x;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (i >= d) return;
+  float g[8], u[8];
+  if constexpr (sizeof(typename T::storage) == 2) {
+    const u16x8 gv = *reinterpret_cast<const u16x8*>(in + t * in_stride + i), uv = *reinterpret_cast<const u16x8*>(in + t * in_stride + d + i);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      g[j] = T::to_f32(gv[j]);
+      u[j] = T::to_f32(uv[j]);
+    }
+    u16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = T::from_f32(clamped_glu_f(g[j], u[j], limit, alpha));
+    *reinterpret_cast<u16x8*>(out + t * (int64_t)d + i) = r;
+  } else {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const f32x4 gv = *reinterpret_cast<const f32x4*>(in + t * in_stride + i + 4 * h);
+      const f32x4 uv = *reinterpret_cast<const f32x4*>(in + t * in_stride + d + i + 4 * h);
+      f32x4 r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = clamped_glu_f(gv[j], uv[j], limit, alpha);
+      *reinterpret_cast<f32x4*>(out + t * (int64_t)d + i + 4 * h) = r;
+    }
+  }
+}
+
 }  // namespace aphro
 
 using namespace aphro;
@@ -667,10 +699,15 @@ extern "C" int aphro_clamped_glu(void* out, const void* in, int64_t in_stride, i
   if (num_tokens == 0) return APHRO_OK;
   APHRO_CHECK(out && in && d > 0 && in_stride >= 2 * (int64_t)d && num_tokens <= 0x7fffffff && (d + 255) / 256 <= 65535,
               "clamped_glu: bad arguments");
+  const bool vec = d % 8 == 0 && in_stride % 8 == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0;
   MIX_DISPATCH_DTYPE(dtype, {
     typedef typename T::storage S;
-    hipLaunchKernelGGL((clamped_glu_kernel<T>), dim3((unsigned)num_tokens, (unsigned)((d + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, (S*)out, (const S*)in, in_stride, d, limit, alpha);
+    if (vec)
+      hipLaunchKernelGGL((clamped_glu_vec8_kernel<T>), dim3((unsigned)num_tokens, (unsigned)((d / 8 + 255) / 256)), dim3(256), 0,
+                         (hipStream_t)stream, (S*)out, (const S*)in, in_stride, d, limit, alpha);
+    else
+      hipLaunchKernelGGL((clamped_glu_kernel<T>), dim3((unsigned)num_tokens, (unsigned)((d + 255) / 256)), dim3(256), 0,
+                         (hipStream_t)stream, (S*)out, (const S*)in, in_stride, d, limit, alpha);
   });
   APHRO_LAUNCH_CHECK();
   return APHRO_OK;
