@@ -66,7 +66,8 @@ def cmd_trace(args) -> int:
         else:
             torch.cuda.synchronize()
         for rid in step.get("end") or []:
-            engine.release(str(rid))
+            if str(rid) in engine.requests:        # a request that never brought a token holds nothing
+                engine.release(str(rid))
         sys.stdout.write("done %s\n" % step["step"])
         sys.stdout.flush()
     return 0

@@ -52,17 +52,20 @@ constexpr int LF_BM = 64, LF_BN = 64;
 // A thread brings in 16-byte chunks cl, cl + 16, ... of ONE pair of neighbouring keys (pair = tid / 16, cl = tid % 16): sixteen
 // lanes fetch 256 contiguous bytes, and a tile costs a thread two block-table lookups.
 // The transposed copy of a tile: column col of the latent is a row of LF_VS dwords (64 keys and padding) at row number
-// (col & 7) * JS + (col >> 3), LF_VS = 4 mod 32 and JS odd.  A store instruction writes one dword per lane for 16 chunks x 4
-// key pairs -- 4 cl + pair: two lanes per bank, the minimum -- and the value-operand reads of 16 columns x 4 key groups x 2
-// dwords land on every bank equally often.
-constexpr int LF_VS = 36, LF_THREADS = 512, LF_CL = 16;
+// (col & 7) * JS + (col >> 3), LF_VS = 34 and JS = 2 mod 16.  What the counters say about the LDS (32 banks of 4 bytes): a 4-byte
+// access is served 32 lanes at a time, an 8-byte one 16 lanes, a 16-byte one 8 lanes.  A transposed store writes one dword per
+// lane for 16 chunks x 2 key pairs per pass -- bank 2 cl + pair: all 32 distinct; an 8-byte value-operand read of the 16
+// columns of a lane group finds them in rows 2 (c & 7) + (c >> 3) mod 16, that is in 16 different bank pairs.  (With 36-dword
+// rows and JS odd, SQ_LDS_BANK_CONFLICT was 0.31 of the LDS cycles.)  The row-major copy XORs the chunk index with key & 7: the
+// 8 keys of a 16-byte fragment read pass hit 8 different bank quads.
+constexpr int LF_VS = 34, LF_THREADS = 512, LF_CL = 16;
 
 template <int R, int P>
 struct LFGeom {
   static constexpr int D = R + P, DP = (D + 31) / 32 * 32, NCH = DP / 8, NKS = DP / 32, NDT = R / 16;
   static constexpr int SWZ = ((NCH & -NCH) - 1) & 7;       // chunk index ^ (key & SWZ): fragment reads spread over the banks
   static constexpr int NI = (NCH + LF_CL - 1) / LF_CL, NDH = NDT / 2;
-  static constexpr int JS = (R / 8) | 1;
+  static constexpr int JS = (R / 8 + 13) / 16 * 16 + 2;
   static constexpr size_t LDS_BYTES = (size_t)LF_BN * DP * sizeof(uint16_t) + (size_t)8 * JS * LF_VS * sizeof(uint32_t);
 };
 
@@ -203,7 +206,7 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
       s[h] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < G::NKS; ++ks) {
-        // chunk (4 ks + g) ^ (key & SWZ) = 8 (ks / 2) + (((ks & 1) * 4 + g) ^ (c & SWZ)): two lane offsets, the rest is immediate
+        // chunk (4 ks + g) ^ swz(key) = 8 (ks / 2) + (((ks & 1) * 4 + g) ^ swz(c)): two lane offsets, the rest is immediate
         const u32x4 kf = *reinterpret_cast<const u32x4*>(krow[ks & 1] + (16 * h) * G::DP + 64 * (ks >> 1));
         s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[h], 0, 0, 0);
       }
@@ -247,7 +250,8 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
 #pragma unroll
       for (int dt = 0; dt < G::NDH; ++dt) {
         const uint32_t* vr = vrow + 2 * dt * LF_VS + 16 * pk;
-        const u32x4 vf = {vr[0], vr[1], vr[8], vr[9]};
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(vr), hi = *reinterpret_cast<const u32x2*>(vr + 8);
+        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[pk]), o[dt], 0, 0, 0);
       }
     }
