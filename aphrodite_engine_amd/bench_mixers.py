@@ -79,7 +79,7 @@ def fekotar_config(s):
            "router": {"experts": FEK_EXPERTS, "top": FEK_TOP, "scale": 1.0, "groups": {"count": FEK_GROUPS, "keep": FEK_KEEP}}}
     layers = [{"type": "latent_attention", "mixer": dict(mixer), "mlp": dense if i == 0 else moe} for i in range(LAYERS)]
     return {"architecture": "Fekotar", "vocab": VOCAB, "width": s["width"], "norm": {"eps": 1e-6}, "logit_scale": 1.0,
-            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": layers}
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 131, "mul_cur": 3}}, "layers": layers}
 
 
 def timed(fn, iters=10, warmup=3):
@@ -425,7 +425,7 @@ def fekotar_kernel_section(s, prompt_len, batch, ctx, device):
         table, pair = torch.randn(VOCAB, W, device=device, dtype=bf), torch.randn(65522, W, device=device, dtype=bf)
         tstate = torch.zeros(batch, dtype=torch.int32, device=device)
         sec = timed(lambda: mops.hashed_pair_embed(table, pair, b.input_ids, tstate, b.state_slots, b.q_start, b.q_len, b.ctx_len,
-                                                   b.seq_of_token, 31, 7))
+                                                   b.seq_of_token, 131, 3))
         rec("hashed_pair_embed_" + name, sec, bytes_=T * W * 8)
         # ---- experts: route, sort, both products, combine -- against the dense feed-forward's library products of equal active size
         h = torch.randn(T, W, device=device, dtype=bf)

@@ -60,8 +60,10 @@ __global__ void latent_prep_kernel(typename T::storage* __restrict__ cq, typenam
     float v = T::to_f32(kr[i]);
     if (i < 2 * half) {
       const int f = i < half ? i : i - half;
-      const float a = pos * inv_freq[f];
-      const float c = cosf(a) * mscale, sn = sinf(a) * mscale;
+      float c, sn;
+      sincosf(pos * inv_freq[f], &sn, &c);
+      c *= mscale;
+      sn *= mscale;
       const float other = T::to_f32(kr[i < half ? i + half : i - half]);
       v = i < half ? v * c - other * sn : v * c + other * sn;
     }
@@ -121,8 +123,10 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     float v = T::to_f32(qr[i]);
     if (i < 2 * half) {
       const int f = i < half ? i : i - half;
-      const float a = (float)pos * inv_freq[f];
-      const float c = cosf(a) * mscale, sn = sinf(a) * mscale;
+      float c, sn;
+      sincosf((float)pos * inv_freq[f], &sn, &c);
+      c *= mscale;
+      sn *= mscale;
       const float other = T::to_f32(qr[i < half ? i + half : i - half]);
       v = i < half ? v * c - other * sn : v * c + other * sn;
     }

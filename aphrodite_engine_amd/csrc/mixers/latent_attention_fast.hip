@@ -150,6 +150,10 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   constexpr float LOG2E = 1.4426950408889634f;
   const float qs = p.scale * LOG2E;
 
+  const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
+  LFStage<R, P> st;                                         // the first tile is on its way while the query operand is made
+  if (t_begin < t_end) lf_load<R, P>(st, p, bt, t_begin, t_end);
+
   // the query operand: [q_lat | rotate(q_rot) | zeros]
   u32x4 qf[G::NKS];
   {
@@ -171,8 +175,10 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
         float o[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const float a = (float)qpos * p.inv_freq[f0 + j];
-          const float cs = cosf(a) * p.mscale, sn = sinf(a) * p.mscale;
+          float cs, sn;
+          sincosf((float)qpos * p.inv_freq[f0 + j], &sn, &cs);
+          cs *= p.mscale;
+          sn *= p.mscale;
           const float x = BFloat::to_f32(mine[j]), y = BFloat::to_f32(other[j]);
           o[j] = low ? x * cs - y * sn : x * cs + y * sn;
         }
@@ -185,15 +191,12 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
 #pragma unroll
   for (int i = 0; i < G::NDH; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -1e30f, l_run = 0.f;
-  const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
   const int kmax = min(qpos, t_end - 1);                    // the last key this row takes from this workgroup's share
 
   const uint16_t* krow[2] = {k_lds + c * G::DP + 8 * (g ^ (c & G::SWZ)), k_lds + c * G::DP + 8 * ((4 | g) ^ (c & G::SWZ))};
   const uint32_t* vrow = vt_lds + ((c & 7) * G::JS + (c >> 3) + 2 * G::NDH * half) * LF_VS + 2 * g;
   const bool idle = r0 + 16 * wave >= nrows;                // a wave without rows only helps to move the tiles
 
-  LFStage<R, P> st;
-  if (t_begin < t_end) lf_load<R, P>(st, p, bt, t_begin, t_end);
   for (int t0 = t_begin; t0 < t_end; t0 += LF_BN) {
     __syncthreads();                                        // the previous tile is consumed
     lf_store<R, P>(st, k_lds, vt_lds);
