@@ -5,11 +5,10 @@
 // query rows of a segment are flattened: row = token * heads + head.  A workgroup of eight waves owns 64 consecutive rows: a
 // PAIR of waves shares 16 rows -- with 16 heads that is one token's heads -- both compute the rows' scores, each accumulates
 // one half of the R output columns (two waves per SIMD hide each other's LDS latency, and half the accumulators leave
-// registers for fragments in flight).  The workgroup walks the visible keys 64 at a time:
+// registers for fragments in flight).  The workgroup walks the visible keys 32 at a time:
 // the tile's cache rows come in with 16-byte loads, go to LDS once row-major (chunk-swizzled: the key operand) and, their
-// first R numbers, once transposed (the value operand; a layout both its stores and its reads pass without bank conflicts beyond
-// the unavoidable); the next tile's rows are fetched into registers while the current
-// tile's products run.  S^T = K Q^T on v_mfma_f32_16x16x32_bf16, so that the probabilities come out in the B-operand layout
+// first R numbers, once transposed (the value operand; layouts both their stores and their reads pass without bank conflicts);
+// tiles alternate between two homes in LDS and the tile after the next is on its way in registers.  S^T = K Q^T on v_mfma_f32_16x16x32_bf16, so that the probabilities come out in the B-operand layout
 // of O^T = C^T P^T; mask and online softmax (base 2) are fp32 on the accumulators.  The query operand is [q_lat | rotate(q_r)]
 // padded with zeros to a multiple of 32, built once per workgroup (the rotation in fp32 at the row's position).
 //
@@ -48,25 +47,28 @@ __device__ __forceinline__ int la_slot(const LAParams& p, const int32_t* bt, int
   return blk * p.block_size + off;
 }
 
-constexpr int LF_BM = 64, LF_BN = 64;
-// A thread brings in 16-byte chunks cl, cl + 16, ... of ONE pair of neighbouring keys (pair = tid / 16, cl = tid % 16): sixteen
-// lanes fetch 256 contiguous bytes, and a tile costs a thread two block-table lookups.
-// The transposed copy of a tile: column col of the latent is a row of LF_VS dwords (64 keys and padding) at row number
-// (col & 7) * JS + (col >> 3), LF_VS = 34 and JS = 2 mod 16.  What the counters say about the LDS (32 banks of 4 bytes): a 4-byte
-// access is served 32 lanes at a time, an 8-byte one 16 lanes, a 16-byte one 8 lanes.  A transposed store writes one dword per
-// lane for 16 chunks x 2 key pairs per pass -- bank 2 cl + pair: all 32 distinct; an 8-byte value-operand read of the 16
-// columns of a lane group finds them in rows 2 (c & 7) + (c >> 3) mod 16, that is in 16 different bank pairs.  (With 36-dword
-// rows and JS odd, SQ_LDS_BANK_CONFLICT was 0.31 of the LDS cycles.)  The row-major copy XORs the chunk index with key & 7: the
-// 8 keys of a 16-byte fragment read pass hit 8 different bank quads.
-constexpr int LF_VS = 34, LF_THREADS = 512, LF_CL = 16;
+constexpr int LF_BM = 64, LF_BN = 32;
+// A thread brings in 16-byte chunks cl, cl + 32, ... of ONE pair of neighbouring keys (pair = tid / 32, cl = tid % 32): 32 lanes
+// fetch 512 contiguous bytes, and a tile costs a thread two block-table lookups.  A tile has TWO homes in LDS: while the waves
+// multiply from one, the next tile is stored into the other -- one barrier per tile, and one wave's stores run beside
+// another's products.
+// The transposed copy of a tile: column col of the latent is a row of LF_VS dwords (32 keys and one dword of padding) at row
+// number (col & 7) * JS + (col >> 3), LF_VS = 17 and JS = 4 mod 32.  What the counters say about the LDS (32 banks of 4 bytes): a
+// 4-byte access is served 32 lanes at a time, a 16-byte one 8 lanes.  A transposed store writes one dword per lane for 32
+// consecutive chunks of one key pair per pass -- bank 17 cl: all 32 distinct; a 4-byte value-operand read of two lane groups
+// finds its 16 columns x 2 key groups in banks 4 (c & 7) + 17 (c >> 3) + 2 g: all 32 distinct.  (Layouts that broke these rules
+// showed SQ_LDS_BANK_CONFLICT at 0.31 of the LDS cycles.)  The row-major copy XORs the chunk index with key & 7: the 8 keys of a
+// 16-byte fragment read pass hit 8 different bank quads.
+constexpr int LF_VS = 17, LF_THREADS = 512, LF_CL = 32;
 
 template <int R, int P>
 struct LFGeom {
   static constexpr int D = R + P, DP = (D + 31) / 32 * 32, NCH = DP / 8, NKS = DP / 32, NDT = R / 16;
   static constexpr int SWZ = ((NCH & -NCH) - 1) & 7;       // chunk index ^ (key & SWZ): fragment reads spread over the banks
   static constexpr int NI = (NCH + LF_CL - 1) / LF_CL, NDH = NDT / 2;
-  static constexpr int JS = (R / 8 + 13) / 16 * 16 + 2;
-  static constexpr size_t LDS_BYTES = (size_t)LF_BN * DP * sizeof(uint16_t) + (size_t)8 * JS * LF_VS * sizeof(uint32_t);
+  static constexpr int JS = (R / 8 + 27) / 32 * 32 + 4;
+  static constexpr int KBUF = LF_BN * DP, VBUF = 8 * JS * LF_VS;         // one home: elements of the row-major copy, dwords of the other
+  static constexpr size_t LDS_BYTES = 2 * ((size_t)KBUF * sizeof(uint16_t) + (size_t)VBUF * sizeof(uint32_t));
 };
 
 template <int R, int P>
@@ -99,7 +101,7 @@ __device__ __forceinline__ void lf_store(const LFStage<R, P>& st, uint16_t* k_ld
   typedef LFGeom<R, P> G;
   const int tp = threadIdx.x / LF_CL, c8 = threadIdx.x % LF_CL;
   const int ta = 2 * tp, tb = 2 * tp + 1;
-  uint16_t* ka = k_lds + ta * G::DP + 8 * (c8 ^ (ta & G::SWZ));      // chunk c8 + 16 it: the swizzle stays within the low 3 bits
+  uint16_t* ka = k_lds + ta * G::DP + 8 * (c8 ^ (ta & G::SWZ));      // chunk c8 + 32 it: the swizzle stays within the low 3 bits
   uint16_t* kb = k_lds + tb * G::DP + 8 * (c8 ^ (tb & G::SWZ));
   uint32_t* vt = vt_lds + c8 * LF_VS + tp;
 #pragma unroll
@@ -124,8 +126,8 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   typedef LFGeom<R, P> G;
   constexpr int NH = LF_BN / 16, NPK = LF_BN / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t la_lds[];
-  uint16_t* k_lds = la_lds;
-  uint32_t* vt_lds = reinterpret_cast<uint32_t*>(la_lds + LF_BN * G::DP);
+  uint16_t* k_lds = la_lds;                                                     // two homes of KBUF elements
+  uint32_t* vt_lds = reinterpret_cast<uint32_t*>(la_lds + 2 * G::KBUF);          // two homes of VBUF dwords
   // waves 2 k and 2 k + 1 share row group k: a launch with one row group (decoded tokens of 16 heads) still uses two SIMDs
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 7, half = (threadIdx.x >> 6) & 1, g = lane >> 4, c = lane & 15;
   const int seq = blockIdx.y, z = blockIdx.z;
@@ -151,8 +153,12 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   const float qs = p.scale * LOG2E;
 
   const int32_t* bt = p.block_tables + (int64_t)seq * p.max_blocks;
-  LFStage<R, P> st;                                         // the first tile is on its way while the query operand is made
-  if (t_begin < t_end) lf_load<R, P>(st, p, bt, t_begin, t_end);
+  LFStage<R, P> st;                                         // the first tiles are on their way while the query operand is made
+  if (t_begin < t_end) {
+    lf_load<R, P>(st, p, bt, t_begin, t_end);
+    lf_store<R, P>(st, k_lds, vt_lds);
+    if (t_begin + LF_BN < t_end) lf_load<R, P>(st, p, bt, t_begin + LF_BN, t_end);
+  }
 
   // the query operand: [q_lat | rotate(q_rot) | zeros]
   u32x4 qf[G::NKS];
@@ -197,12 +203,11 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   const uint32_t* vrow = vt_lds + ((c & 7) * G::JS + (c >> 3) + 2 * G::NDH * half) * LF_VS + 2 * g;
   const bool idle = r0 + 16 * wave >= nrows;                // a wave without rows only helps to move the tiles
 
-  for (int t0 = t_begin; t0 < t_end; t0 += LF_BN) {
-    __syncthreads();                                        // the previous tile is consumed
-    lf_store<R, P>(st, k_lds, vt_lds);
-    __syncthreads();
-    if (t0 + LF_BN < t_end) lf_load<R, P>(st, p, bt, t0 + LF_BN, t_end);       // in flight during this tile's products
-    if (idle || t0 > wpos_hi) continue;                     // every key of the tile is ahead of the wave's rows
+  int cur = 0;
+  __syncthreads();
+  for (int t0 = t_begin; t0 < t_end; t0 += LF_BN, cur ^= 1) {
+   if (!(idle || t0 > wpos_hi)) {                           // else: every key of the tile is ahead of the wave's rows
+    const int kofs = cur * G::KBUF, vofs = cur * G::VBUF;
     f32x4 s[NH];
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
@@ -210,7 +215,7 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
 #pragma unroll
       for (int ks = 0; ks < G::NKS; ++ks) {
         // chunk (4 ks + g) ^ swz(key) = 8 (ks / 2) + (((ks & 1) * 4 + g) ^ swz(c)): two lane offsets, the rest is immediate
-        const u32x4 kf = *reinterpret_cast<const u32x4*>(krow[ks & 1] + (16 * h) * G::DP + 64 * (ks >> 1));
+        const u32x4 kf = *reinterpret_cast<const u32x4*>(krow[ks & 1] + kofs + (16 * h) * G::DP + 64 * (ks >> 1));
         s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[h], 0, 0, 0);
       }
     }
@@ -252,12 +257,17 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
     for (int pk = 0; pk < NPK; ++pk) {
 #pragma unroll
       for (int dt = 0; dt < G::NDH; ++dt) {
-        const uint32_t* vr = vrow + 2 * dt * LF_VS + 16 * pk;
-        const u32x2 lo = *reinterpret_cast<const u32x2*>(vr), hi = *reinterpret_cast<const u32x2*>(vr + 8);
-        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+        const uint32_t* vr = vrow + vofs + 2 * dt * LF_VS + 16 * pk;
+        const u32x4 vf = {vr[0], vr[1], vr[8], vr[9]};
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf[pk]), o[dt], 0, 0, 0);
       }
     }
+   }
+    if (t0 + LF_BN < t_end) {                               // the next tile goes to the other home, the one after it is requested
+      lf_store<R, P>(st, k_lds + (cur ^ 1) * G::KBUF, vt_lds + (cur ^ 1) * G::VBUF);
+      if (t0 + 2 * LF_BN < t_end) lf_load<R, P>(st, p, bt, t0 + 2 * LF_BN, t_end);
+    }
+    __syncthreads();
   }
   float l = l_run;
   l += __shfl_xor(l, 16, 64);
