@@ -18,8 +18,8 @@
 namespace aphro {
 
 constexpr int LA_WAVES = 4;
-constexpr int LA_MAX_DIM = 1024;        // R + P
-constexpr int LA_MAX_EPL = 8;           // R <= 512
+constexpr int LA_MAX_DIM = 2048;        // R + P
+constexpr int LA_MAX_EPL = 16;          // R <= 1024
 
 template <typename T>
 __global__ void latent_prep_kernel(typename T::storage* __restrict__ cq, typename T::storage* __restrict__ cache,
@@ -293,7 +293,9 @@ extern "C" int aphro_latent_attention_plain(void* out, int64_t out_stride, int64
       case 3: LA_LAUNCH(3); break;
       case 4: LA_LAUNCH(4); break;
       case 5: case 6: LA_LAUNCH(6); break;
-      default: LA_LAUNCH(8); break;
+      case 7: case 8: LA_LAUNCH(8); break;
+      case 9: case 10: case 11: case 12: LA_LAUNCH(12); break;
+      default: LA_LAUNCH(16); break;
     }
   });
 #undef LA_LAUNCH

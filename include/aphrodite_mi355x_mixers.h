@@ -228,7 +228,7 @@ int aphro_latent_prep(void* cq, void* cache, int64_t num_cache_rows, const void*
                       int rot_dim, int rot_dims, float eps, int dtype, void* stream);
 /* Causal softmax attention of every head over the shared latent rows cache [blocks, block, kv_rank + rot_dim]:
  * score = ([q_lat | rotate(q_rot)] . row) * scale, out = sum p * row[:kv_rank].  q_lat / q_rot / out are addressed as
- * base + t * stride + head * head_stride (elements); any sizes (kv_rank <= 512), fp32 math. */
+ * base + t * stride + head * head_stride (elements); any sizes (kv_rank <= 1024), fp32 math. */
 int aphro_latent_attention_plain(void* out, int64_t out_stride, int64_t out_head_stride, const void* q_lat, int64_t ql_stride,
                                  int64_t ql_head_stride, const void* q_rot, int64_t qr_stride, int64_t qr_head_stride,
                                  const void* cache, const int32_t* block_tables, int max_blocks, int64_t num_blocks, int block_size,
