@@ -179,7 +179,7 @@ MIXERS_SIGNATURES = {
     "aphro_depth_residual_rms_norm": (I, [P, P, P, L, P, L, I, P, F, P, P, L, I, F, I, P]),
     "aphro_poly_norm": (I, [P, P, L, L, I, F, F, F, F, F, I, P]),
     "aphro_differential_norm_gate": (I, [P, L, P, L, P, L, L, I, I, I, F, F, F, I, P]),
-    "aphro_short_conv": (I, [P, L, P, P, P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, I, I, P]),
+    "aphro_short_conv": (I, [P, L, P, P, P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, P]),
     "aphro_windowed_attention": (I, [P, L, P, L, P, P, P, I, L, I, P, P, P, P, L, I, I, I, I, I, I, I, I, F, I, I, I, P, L, I, P]),
     "aphro_differential_window_attention_supported": (I, [I, I, I, I, I]),
     "aphro_differential_window_attention": (I, [P, L, P, L, P, L, P, P, P, I, L, I, P, P, P, P, L, I, I, I, I, I, I, I, F, I, I, F, F,
@@ -196,12 +196,18 @@ MIXERS_SIGNATURES = {
     "aphro_token_state_write": (I, [P, P, P, P, P, I, P]),
     "aphro_residual_add2_rms_norm": (I, [P, P, L, P, L, P, P, P, L, I, F, I, P]),
     "aphro_latent_prep": (I, [P, P, L, P, L, I, I, P, P, P, P, P, P, P, F, L, I, I, I, I, F, I, P]),
-    "aphro_latent_attention_plain": (I, [P, L, L, P, L, L, P, L, L, P, P, I, L, I, P, P, P, P, F, L, I, I, I, I, F, I, P]),
+    "aphro_latent_attention_plain": (I, [P, L, L, P, L, L, P, L, L, P, P, I, L, I, P, P, P, P, F, L, I, I, I, I, F, I, P, I, P]),
     "aphro_latent_attention_fast_supported": (I, [I, I, I, I]),
     "aphro_latent_attention_splits": (I, [L, I, I, I, I]),
-    "aphro_latent_attention": (I, [P, L, L, P, L, L, P, L, L, P, P, I, L, I, P, P, P, P, P, F, L, I, I, I, I, I, I, I, F, P, L, I, P]),
+    "aphro_latent_attention": (I, [P, L, L, P, L, L, P, L, L, P, P, I, L, I, P, P, P, P, P, F, L, I, I, I, I, I, I, I, F, I, P, P, L, I, P]),
     "aphro_sigmoid_gate_mul": (I, [P, L, P, L, P, L, L, I, I, P]),
     "aphro_experts_route_grouped": (I, [P, P, P, L, I, I, I, I, I, F, P]),
+    "aphro_experts_route_topk": (I, [P, P, P, P, L, I, I, P]),
+    "aphro_hyper_residual_rms_norm": (I, [P, P, L, P, P, P, F, P, P, P, P, L, I, I, F, I, P]),
+    "aphro_logit_softcap": (I, [P, P, L, F, F, I, P]),
+    "aphro_gated_delta_scan": (I, [P, P, L, P, L, P, L, P, L, P, L, P, P, P, P, I, P, P, P, I, L, I, I, I, I, F, F, I, I, P]),
+    "aphro_gated_head_rms_norm": (I, [P, L, P, P, P, L, L, I, I, F, I, I, P]),
+    "aphro_rotary_qk_norm_kv_write": (I, [P, L, P, P, P, L, P, L, P, L, P, L, P, L, F, P, P, P, P, L, I, I, I, I, I, I, I, F, I, P]),
 }
 
 OK = 0

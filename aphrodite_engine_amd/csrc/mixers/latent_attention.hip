@@ -9,7 +9,8 @@
 //   latent_prep        per token: RMS norm of the query latent -> [T, q_rank]; RMS norm of the key/value latent and the rotation
 //                      of the shared key part at the token's position -> the cache row at its slot
 //   latent_attention   any sizes, fp32 math: a workgroup of four waves per (row, head); lane = key for the scores, lane =
-//                      column for P C; rotates the query's rotary part on load
+//                      column for P C; rotates the query's rotary part on load; optional sliding window (row i sees key j
+//                      with 0 <= i - j < window) and per-head sink (exp(sink) joins the softmax denominator, unscaled)
 //   sigmoid_gate_mul   out = x * sigmoid(gate), elementwise
 // Rotation ("rotate half" over the first rot_dims numbers of the rotary part): the pair (u, v) = (x[i], x[i + rot_dims / 2])
 // becomes (u cos a - v sin a, v cos a + u sin a) * mscale with a = position * inv_freq[i], all in fp32.
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     const typename T::storage* __restrict__ cache, const int32_t* __restrict__ block_tables, int max_blocks, int64_t num_blocks,
     int block_size, const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ seq_of_token, const float* __restrict__ inv_freq, float mscale, int kv_rank, int rot_dim,
-    int rot_dims, float scale) {
+    int rot_dims, float scale, int window, const float* __restrict__ sink) {
   __shared__ __attribute__((aligned(16))) float qsh[LA_MAX_DIM];
   __shared__ float merge[LA_WAVES][2 + EPL * 64];
   const int t = blockIdx.x, h = blockIdx.y;
@@ -138,11 +139,12 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
 #pragma unroll
   for (int c = 0; c < EPL; ++c) acc[c] = 0.f;
   const int n = pos + 1;
+  const int first = window > 0 ? max(0, n - window) : 0;     // the oldest key the row sees
   const int ntiles = (n + 63) >> 6;
-  for (int tile = wave; tile < ntiles; tile += LA_WAVES) {
+  for (int tile = (first >> 6) + wave; tile < ntiles; tile += LA_WAVES) {
     const int j = tile * 64 + lane;
     float sc = -INFINITY;
-    if (j < n) {
+    if (j < n && j >= first) {
       const int blk = bt[j / block_size];
       if (blk >= 0 && blk < num_blocks) sc = la_dot<T>(qsh, cache + ((int64_t)blk * block_size + j % block_size) * dim, dim) * scale;
     }
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     for (int c = 0; c < EPL; ++c) acc[c] *= alpha;
     const int cnt = min(64, n - tile * 64);
 #pragma unroll 4
-    for (int jj = 0; jj < cnt; ++jj) {
+    for (int jj = max(0, first - tile * 64); jj < cnt; ++jj) {
       const float pj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, p), jj));
       const int j2 = tile * 64 + jj;
       int blk = bt[j2 / block_size];
@@ -176,10 +178,10 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
   for (int c = 0; c < EPL; ++c) merge[wave][2 + lane + 64 * c] = acc[c];
   __syncthreads();
   if (wave != 0) return;
-  float M = -INFINITY;
+  float M = sink ? sink[h] : -INFINITY;                      // the sink: one more term of the denominator, no value
 #pragma unroll
   for (int w = 0; w < LA_WAVES; ++w) M = fmaxf(M, merge[w][0]);
-  float L = 0.f, f[LA_WAVES];
+  float L = sink ? expf(sink[h] - M) : 0.f, f[LA_WAVES];
 #pragma unroll
   for (int w = 0; w < LA_WAVES; ++w) {
     f[w] = (merge[w][0] == -INFINITY) ? 0.f : expf(merge[w][0] - M);
@@ -268,8 +270,8 @@ extern "C" int aphro_latent_attention_plain(void* out, int64_t out_stride, int64
                                             int64_t qr_head_stride, const void* cache, const int32_t* block_tables, int max_blocks,
                                             int64_t num_blocks, int block_size, const int32_t* q_start, const int32_t* ctx_len,
                                             const int32_t* seq_of_token, const float* inv_freq, float mscale, int64_t num_tokens,
-                                            int heads, int kv_rank, int rot_dim, int rot_dims, float scale, int dtype,
-                                            void* stream) {
+                                            int heads, int kv_rank, int rot_dim, int rot_dims, float scale, int window,
+                                            const float* sink, int dtype, void* stream) {
   if (num_tokens == 0) return APHRO_OK;
   APHRO_CHECK(out && q_lat && (q_rot || rot_dim == 0) && cache && block_tables && q_start && ctx_len && seq_of_token &&
                   (rot_dims == 0 || inv_freq), "latent_attention: null argument");
@@ -284,7 +286,7 @@ extern "C" int aphro_latent_attention_plain(void* out, int64_t out_stride, int64
   hipLaunchKernelGGL((latent_attention_kernel<T, EPL>), grid, dim3(256), 0, (hipStream_t)stream, (S*)out, out_stride,           \
                      out_head_stride, (const S*)q_lat, ql_stride, ql_head_stride, (const S*)q_rot, qr_stride, qr_head_stride,   \
                      (const S*)cache, block_tables, max_blocks, num_blocks, block_size, q_start, ctx_len, seq_of_token, inv_freq, \
-                     mscale, kv_rank, rot_dim, rot_dims, scale)
+                     mscale, kv_rank, rot_dim, rot_dims, scale, window, sink)
   MIX_DISPATCH_DTYPE(dtype, {
     typedef typename T::storage S;
     switch (epl) {

@@ -28,6 +28,8 @@ struct LAParams {
   const int32_t* q_len;
   const int32_t* ctx_len;
   const float* inv_freq;
+  const float* sink;  // fp32 [heads] or NULL
+  int window;         // <= 0: none
   int64_t out_stride, out_head_stride, ql_stride, ql_head_stride, qr_stride, qr_head_stride, num_blocks;
   int max_blocks, block_size, bs_shift, heads, nsplit;
   float scale, mscale;
@@ -147,8 +149,10 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   const int wpos_lo = ctx + wrow_lo / H, wpos_hi = ctx + wrow_hi / H;
   const int nk = ctx + min(r0 + LF_BM - 1, nrows - 1) / H + 1;          // keys the workgroup's last row sees
   // this workgroup's share of the key tiles
-  const int tiles = (nk + LF_BN - 1) / LF_BN, per = (tiles + p.nsplit - 1) / p.nsplit;
-  const int t_begin = z * per * LF_BN, t_end = min(nk, (z + 1) * per * LF_BN);
+  // under a window the walk starts at the tile of the oldest key the workgroup's first row sees
+  const int k_first = p.window > 0 ? max(0, ctx + r0 / H - p.window + 1) / LF_BN * LF_BN : 0;
+  const int tiles = (nk - k_first + LF_BN - 1) / LF_BN, per = (tiles + p.nsplit - 1) / p.nsplit;
+  const int t_begin = k_first + z * per * LF_BN, t_end = min(nk, k_first + (z + 1) * per * LF_BN);
   constexpr float LOG2E = 1.4426950408889634f;
   const float qs = p.scale * LOG2E;
 
@@ -198,6 +202,8 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   for (int i = 0; i < G::NDH; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -1e30f, l_run = 0.f;
   const int kmax = min(qpos, t_end - 1);                    // the last key this row takes from this workgroup's share
+  const int kmin = p.window > 0 ? qpos - p.window + 1 : 0;  // the oldest key this row sees (may be negative)
+  const int wmin_lo = p.window > 0 ? wpos_lo - p.window + 1 : 0, wmin_hi = p.window > 0 ? wpos_hi - p.window + 1 : 0;
 
   const uint16_t* krow[2] = {k_lds + c * G::DP + 8 * (g ^ (c & G::SWZ)), k_lds + c * G::DP + 8 * ((4 | g) ^ (c & G::SWZ))};
   const uint32_t* vrow = vt_lds + ((c & 7) * G::JS + (c >> 3) + 2 * G::NDH * half) * LF_VS + 2 * g;
@@ -206,7 +212,7 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   int cur = 0;
   __syncthreads();
   for (int t0 = t_begin; t0 < t_end; t0 += LF_BN, cur ^= 1) {
-   if (!(idle || t0 > wpos_hi)) {                           // else: every key of the tile is ahead of the wave's rows
+   if (!(idle || t0 > wpos_hi || t0 + LF_BN <= wmin_lo)) {  // else: every key of the tile is ahead of the wave's rows or behind their windows
     const int kofs = cur * G::KBUF, vofs = cur * G::VBUF;
     f32x4 s[NH];
 #pragma unroll
@@ -219,7 +225,7 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
         s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[h], 0, 0, 0);
       }
     }
-    const bool edge = t0 + LF_BN - 1 > min(wpos_lo, t_end - 1);   // some key of the tile is not for some row of the wave
+    const bool edge = t0 + LF_BN - 1 > min(wpos_lo, t_end - 1) || t0 < wmin_hi;   // some key of the tile is not for some row of the wave
     float pv[NH][4];
     float mx = -1e30f;
 #pragma unroll
@@ -227,7 +233,10 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float xv = s[h][r] * qs;
-        if (edge) xv = t0 + 16 * h + 4 * g + r <= kmax ? xv : -1e30f;
+        if (edge) {
+          const int key = t0 + 16 * h + 4 * g + r;
+          xv = (key <= kmax && key >= kmin) ? xv : -1e30f;
+        }
         pv[h][r] = xv;
         mx = fmaxf(mx, xv);
       }
@@ -274,7 +283,11 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
   l += __shfl_xor(l, 32, 64);
   if (!rvalid) return;
   if (p.nsplit == 1) {
-    const float f = l > 0.f ? 1.f / l : 0.f;
+    float f = l > 0.f ? 1.f / l : 0.f;
+    if (p.sink) {                                           // one more term of the denominator: exp(sink), no value
+      const float s2 = p.sink[head] * LOG2E, M = fmaxf(m_run, s2), fo = __builtin_amdgcn_exp2f(m_run - M);
+      f = fo / (l * fo + __builtin_amdgcn_exp2f(s2 - M));
+    }
     uint16_t* op = p.out + (int64_t)(s0 + tok) * p.out_stride + (int64_t)head * p.out_head_stride + 16 * G::NDH * half;
 #pragma unroll
     for (int dt = 0; dt < G::NDH; ++dt)
@@ -296,7 +309,7 @@ __global__ __launch_bounds__(LF_THREADS) void la_mfma_kernel(LAParams p) {
 // split's piece in flight before it adds them up
 constexpr int LA_MAX_SPLIT = 16;
 __global__ void la_merge_kernel(uint16_t* __restrict__ out, int64_t out_stride, int64_t out_head_stride, const float* __restrict__ ws,
-                                int heads, int nsplit, int R) {
+                                int heads, int nsplit, int R, const float* __restrict__ sink) {
   const int64_t t = blockIdx.x;
   const int head = blockIdx.y;
   const float* wp = ws + ((t * heads + head) * nsplit) * (int64_t)(2 + R);
@@ -308,11 +321,12 @@ __global__ void la_merge_kernel(uint16_t* __restrict__ out, int64_t out_stride, 
       ml[zz] = *reinterpret_cast<const f32x2*>(wp + (int64_t)zz * (2 + R));
       v[zz] = col < R ? *reinterpret_cast<const f32x2*>(wp + (int64_t)zz * (2 + R) + 2 + col) : f32x2{0.f, 0.f};
     }
-  float M = -1e30f;
+  const float s2 = sink ? sink[head] * 1.4426950408889634f : -1e30f;
+  float M = s2;
 #pragma unroll
   for (int zz = 0; zz < LA_MAX_SPLIT; ++zz)
     if (zz < nsplit) M = fmaxf(M, ml[zz][0]);
-  float L = 0.f, a0 = 0.f, a1 = 0.f;
+  float L = sink ? __builtin_amdgcn_exp2f(s2 - M) : 0.f, a0 = 0.f, a1 = 0.f;
 #pragma unroll
   for (int zz = 0; zz < LA_MAX_SPLIT; ++zz)
     if (zz < nsplit && ml[zz][1] > 0.f) {
@@ -344,7 +358,7 @@ static int la_launch(const LAParams& p, int num_seqs, int max_q_len, int64_t num
                      stream, p);
   if (p.nsplit > 1)
     hipLaunchKernelGGL(la_merge_kernel, dim3((unsigned)num_tokens, (unsigned)p.heads), dim3((R / 2 + 63) / 64 * 64), 0, stream, p.out,
-                       p.out_stride, p.out_head_stride, p.ws, p.heads, p.nsplit, R);
+                       p.out_stride, p.out_head_stride, p.ws, p.heads, p.nsplit, R, p.sink);
   return APHRO_OK;
 }
 
@@ -357,8 +371,8 @@ extern "C" int aphro_latent_attention_plain(void* out, int64_t out_stride, int64
                                             int64_t qr_head_stride, const void* cache, const int32_t* block_tables, int max_blocks,
                                             int64_t num_blocks, int block_size, const int32_t* q_start, const int32_t* ctx_len,
                                             const int32_t* seq_of_token, const float* inv_freq, float mscale, int64_t num_tokens,
-                                            int heads, int kv_rank, int rot_dim, int rot_dims, float scale, int dtype,
-                                            void* stream);
+                                            int heads, int kv_rank, int rot_dim, int rot_dims, float scale, int window,
+                                            const float* sink, int dtype, void* stream);
 
 #define LA_FAST_SIZES(X) X(128, 16) X(128, 32) X(256, 32) X(256, 64) X(512, 64)
 
@@ -388,7 +402,8 @@ extern "C" int aphro_latent_attention(void* out, int64_t out_stride, int64_t out
                                       int block_size, const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
                                       const int32_t* seq_of_token, const float* inv_freq, float mscale, int64_t num_tokens,
                                       int num_seqs, int max_q_len, int max_kv_len, int heads, int kv_rank, int rot_dim, int rot_dims,
-                                      float scale, float* workspace, int64_t workspace_floats, int dtype, void* stream) {
+                                      float scale, int window, const float* sink, float* workspace, int64_t workspace_floats,
+                                      int dtype, void* stream) {
   if (num_tokens == 0) return APHRO_OK;
   const auto al16 = [](const void* ptr) { return ((uintptr_t)ptr & 15) == 0; };
   const bool fast = aphro_latent_attention_fast_supported(kv_rank, rot_dim, rot_dims, dtype) && q_len && num_seqs > 0 && max_q_len > 0 &&
@@ -398,8 +413,8 @@ extern "C" int aphro_latent_attention(void* out, int64_t out_stride, int64_t out
   if (!fast)
     return aphro_latent_attention_plain(out, out_stride, out_head_stride, q_lat, ql_stride, ql_head_stride, q_rot, qr_stride,
                                         qr_head_stride, cache, block_tables, max_blocks, num_blocks, block_size, q_start, ctx_len,
-                                        seq_of_token, inv_freq, mscale, num_tokens, heads, kv_rank, rot_dim, rot_dims, scale, dtype,
-                                        stream);
+                                        seq_of_token, inv_freq, mscale, num_tokens, heads, kv_rank, rot_dim, rot_dims, scale, window,
+                                        sink, dtype, stream);
   APHRO_CHECK(out && q_lat && q_rot && cache && block_tables && q_start && ctx_len && inv_freq, "latent_attention: null argument");
   APHRO_CHECK(heads > 0 && heads <= 65535 && block_size > 0 && max_blocks > 0 && num_blocks > 0 && num_seqs <= 65535,
               "latent_attention: bad geometry");
@@ -413,6 +428,8 @@ extern "C" int aphro_latent_attention(void* out, int64_t out_stride, int64_t out
   p.q_len = q_len;
   p.ctx_len = ctx_len;
   p.inv_freq = inv_freq;
+  p.sink = sink;
+  p.window = window;
   p.out_stride = out_stride;
   p.out_head_stride = out_head_stride;
   p.ql_stride = ql_stride;

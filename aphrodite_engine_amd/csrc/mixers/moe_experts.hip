@@ -83,6 +83,56 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ id
   }
 }
 
+// Router whose weights are the softmax over the CHOSEN logits only: z + bias, the `top` largest are chosen (ties to the lower
+// index), their weights are exp(z_k - max) / sum over the chosen.  One wave per token.
+__global__ __launch_bounds__(256) void moe_route_topk_kernel(int32_t* __restrict__ ids, float* __restrict__ weights,
+                                                             const float* __restrict__ z, const float* __restrict__ bias,
+                                                             int64_t num_tokens, int outputs, int top) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* ch = lds + (size_t)wave * (outputs + top);
+  float* we = ch + outputs;                     // the chosen logits' exponentials
+  const int64_t tt = (int64_t)blockIdx.x * 4 + wave;
+  const bool live = tt < num_tokens;
+  const int64_t t = live ? tt : num_tokens - 1;
+  const float* zr = z + t * outputs;
+  for (int i = lane; i < outputs; i += 64) ch[i] = zr[i] + (bias ? bias[i] : 0.f);
+  __syncthreads();
+  float first = 0.f, sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = lane; i < outputs; i += 64) {
+      const float v = ch[i];
+      if (v > bv) {
+        bv = v;
+        bi = i;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (bi >= outputs) bi = 0;                // every value was NaN: still a valid index
+    if (k == 0) first = bv;                   // the first chosen is the largest
+    const float e = expf(bv - first);
+    sum += e;
+    if (lane == 0) {
+      if (live) ids[t * top + k] = bi;
+      we[k] = e;
+      ch[bi] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  if (live)
+    for (int k = lane; k < top; k += 64) weights[t * top + k] = we[k] / sum;
+}
+
 // Sigmoid router with a choice limited to the best groups of neighbouring experts; one wave per token.  s = sigmoid(z); a
 // group's score is the sum of its `group_top` largest s; only experts of the `keep` best groups can be chosen; the `top`
 // largest s among those are chosen and weighted by s * scale (not renormalised).  Ties go to the lower index.
@@ -558,6 +608,17 @@ extern "C" int aphro_experts_route(int32_t* ids, float* weights, const float* ro
               "moe_route: %d router outputs (<= 2048), top %d", outputs, top);
   hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((num_tokens + 3) / 4)), dim3(256), (size_t)8 * outputs * sizeof(float),
                      (hipStream_t)stream, ids, weights, router_out, correction, num_tokens, outputs, top);
+  APHRO_LAUNCH_CHECK();
+  return APHRO_OK;
+}
+
+extern "C" int aphro_experts_route_topk(int32_t* ids, float* weights, const float* router_out, const float* bias, int64_t num_tokens,
+                                        int outputs, int top, void* stream) {
+  if (num_tokens == 0) return APHRO_OK;
+  APHRO_CHECK(ids && weights && router_out && outputs > 0 && top > 0 && top <= outputs && outputs <= 2048,
+              "moe_route_topk: %d router outputs (<= 2048), top %d", outputs, top);
+  hipLaunchKernelGGL(moe_route_topk_kernel, dim3((unsigned)((num_tokens + 3) / 4)), dim3(256), (size_t)4 * (outputs + top) * sizeof(float),
+                     (hipStream_t)stream, ids, weights, router_out, bias, num_tokens, outputs, top);
   APHRO_LAUNCH_CHECK();
   return APHRO_OK;
 }

@@ -6,7 +6,7 @@
 //
 // The channels are [q | k | v]: the q part goes to a dense output, the k and v parts straight into the token-major paged
 // cache at the rows' slots (what attention reads is the convolved key and value).  Products and sums are fp32, one rounding
-// to the storage type.
+// to the storage type.  act 1: silu on the convolution's result (fp32, before the rounding).
 #include "mixers_common.h"
 
 namespace aphro {
@@ -21,7 +21,7 @@ __global__ void short_conv_kernel(typename T::storage* __restrict__ q_out, int64
                                   const typename T::storage* __restrict__ w, const typename T::storage* __restrict__ state,
                                   const int32_t* __restrict__ state_slots, const int32_t* __restrict__ q_start,
                                   const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ seq_of_token, int cq, int ck,
-                                  int cv, int taps) {
+                                  int cv, int taps, int act) {
   const int64_t t = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   const int C = cq + ck + cv;
@@ -37,6 +37,7 @@ __global__ void short_conv_kernel(typename T::storage* __restrict__ q_out, int64
     else if (ctx + i >= 0) x = T::to_f32(st[(int64_t)(taps - 1 + i) * C]);
     acc += T::to_f32(w[(int64_t)c * taps + j]) * x;
   }
+  if (act) acc = silu_f(acc);
   const typename T::storage y = T::from_f32(acc);
   if (c < cq) {
     q_out[t * q_out_stride + c] = y;
@@ -84,7 +85,8 @@ __global__ __launch_bounds__(256) void short_conv_vec8_kernel(
     typename T::storage* __restrict__ v_cache, const int64_t* __restrict__ cache_slots, int64_t num_cache_slots,
     const typename T::storage* __restrict__ u, int64_t u_stride, const typename T::storage* __restrict__ w,
     const typename T::storage* __restrict__ state, const int32_t* __restrict__ state_slots, const int32_t* __restrict__ q_start,
-    const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ seq_of_token, int64_t num_tokens, int cq, int ck, int cv) {
+    const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ seq_of_token, int64_t num_tokens, int cq, int ck, int cv,
+    int act) {
   const int c0 = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   const int C = cq + ck + cv;
   if (c0 >= C) return;
@@ -135,6 +137,10 @@ __global__ __launch_bounds__(256) void short_conv_vec8_kernel(
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[i] += wv[j][i] * x[i];
     }
+    if (act) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = silu_f(acc[i]);
+    }
     if (c0 < cq) {
       sc_store8<T>(q_out + t * q_out_stride + c0, acc);
     } else {
@@ -178,12 +184,13 @@ extern "C" int aphro_short_conv(void* q_out, int64_t q_out_stride, void* k_cache
                                 int64_t num_cache_slots, const void* u, int64_t u_stride, const void* w, void* state,
                                 const int32_t* state_slots, const int32_t* q_start, const int32_t* q_len,
                                 const int32_t* ctx_len, const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int cq,
-                                int ck, int cv, int taps, int dtype, void* stream) {
+                                int ck, int cv, int taps, int act, int dtype, void* stream) {
   if (num_tokens == 0) return APHRO_OK;
   const int C = cq + ck + cv;
   APHRO_CHECK(u && w && q_start && q_len && ctx_len && seq_of_token && num_seqs > 0 && cq >= 0 && ck >= 0 && cv >= 0 && C > 0,
               "short_conv: bad arguments");
   APHRO_CHECK(taps >= 1 && taps <= SC_MAX_TAPS, "short_conv: %d taps (1 .. %d)", taps, SC_MAX_TAPS);
+  APHRO_CHECK(act == 0 || act == 1, "short_conv: activation %d (0 none, 1 silu)", act);
   APHRO_CHECK(taps == 1 || (state && state_slots), "short_conv: more than one tap needs the state slots");
   APHRO_CHECK(u_stride >= C && (cq == 0 || (q_out && q_out_stride >= cq)), "short_conv: row strides smaller than the rows");
   APHRO_CHECK(ck + cv == 0 || (k_cache && v_cache && cache_slots && num_cache_slots > 0 && ck > 0 && cv > 0),
@@ -197,7 +204,7 @@ extern "C" int aphro_short_conv(void* q_out, int64_t q_out_stride, void* k_cache
   hipLaunchKernelGGL((short_conv_vec8_kernel<T, TAPS, TOK>), dim3((unsigned)((num_tokens + TOK - 1) / TOK), (unsigned)((C / 8 + 255) / 256)), \
                      dim3(C / 8 >= 256 ? 256 : (C / 8 + 63) / 64 * 64), 0, (hipStream_t)stream, (S*)q_out, q_out_stride, (S*)k_cache,     \
                      (S*)v_cache, cache_slots, num_cache_slots, (const S*)u, u_stride, (const S*)w, (const S*)state, state_slots,        \
-                     q_start, ctx_len, seq_of_token, num_tokens, cq, ck, cv)
+                     q_start, ctx_len, seq_of_token, num_tokens, cq, ck, cv, act)
   MIX_DISPATCH_DTYPE(dtype, {
     typedef typename T::storage S;
     if (vec && taps == 2) SC_VEC(2);
@@ -207,7 +214,7 @@ extern "C" int aphro_short_conv(void* q_out, int64_t q_out_stride, void* k_cache
     hipLaunchKernelGGL((short_conv_kernel<T>), dim3((unsigned)num_tokens, (unsigned)((C + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (S*)q_out, q_out_stride, (S*)k_cache, (S*)v_cache, cache_slots, num_cache_slots,
                        (const S*)u, u_stride, (const S*)w, (const S*)state, state_slots, q_start, ctx_len, seq_of_token, cq, ck,
-                       cv, taps);
+                       cv, taps, act);
     if (taps > 1)
       hipLaunchKernelGGL((short_conv_state_kernel<T>), dim3((unsigned)num_seqs, (unsigned)((C + 255) / 256)), dim3(256), 0,
                          (hipStream_t)stream, (S*)state, (const S*)u, u_stride, state_slots, q_start, q_len, ctx_len, C, taps);

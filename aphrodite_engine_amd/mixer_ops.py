@@ -306,11 +306,11 @@ def differential_norm_gate(out: torch.Tensor, a: torch.Tensor, gate: Optional[to
 def short_conv(u: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], state_slots: torch.Tensor, q_start: torch.Tensor,
                q_len: torch.Tensor, ctx_len: torch.Tensor, seq_of_token: torch.Tensor, cq: int, ck: int = 0, cv: int = 0,
                k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
-               slot_mapping: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+               slot_mapping: Optional[torch.Tensor] = None, act: int = 0) -> Optional[torch.Tensor]:
     """Short causal convolution over time on the channels of u [T, cq + ck + cv] (dense rows, any row stride) with w
     [channels, taps]; returns the first cq channels [T, cq]; the ck and cv channels go into the paged caches
     (k_cache [blocks, block, ck], v_cache [blocks, block, cv] in any further split of the last axis) at ``slot_mapping``.
-    state [slots, taps - 1, channels] holds every request's last inputs and is advanced."""
+    state [slots, taps - 1, channels] holds every request's last inputs and is advanced.  ``act`` 1: silu on the result."""
     _cuda(u, w, state, state_slots, q_start, q_len, ctx_len, seq_of_token, k_cache, v_cache, slot_mapping)
     C = cq + ck + cv
     T, S = u.shape[0], q_start.numel()
@@ -334,8 +334,8 @@ def short_conv(u: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], 
     check(_lib.mixers_lib().aphro_short_conv(
         _p(q), cq, _p(k_cache) if ck + cv else None, _p(v_cache) if ck + cv else None, _p(slot_mapping) if ck + cv else None, ncs,
         u.data_ptr(), _rows(u, C, "short_conv u"), w.data_ptr(), _p(state) if taps > 1 else None, state_slots.data_ptr(),
-        q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), T, S, cq, ck, cv, taps, _dt(u), _stream()),
-        "short_conv")
+        q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), T, S, cq, ck, cv, taps, int(act), _dt(u),
+        _stream()), "short_conv")
     return q
 
 
@@ -582,13 +582,19 @@ def _head_view(t: torch.Tensor, T: int, heads: int, n: int, what: str):
 def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: Optional[torch.Tensor], cache: torch.Tensor,
                      block_tables: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor,
                      seq_of_token: torch.Tensor, q_len_range, inv_freq: Optional[torch.Tensor], mscale: float, rot_dims: int,
-                     scale: float, max_kv_len: int = 0, plain: bool = False) -> None:
+                     scale: float, max_kv_len: int = 0, plain: bool = False, window: int = 0,
+                     sink: Optional[torch.Tensor] = None) -> None:
     """Causal softmax attention of a batch of segments over latent cache rows [c | k_r] that all heads share.  q_lat
     [T, heads, kv_rank] (every head's query carried into the latent), q_rot [T, heads, rot_dim] (raw: rotated here at the row's
     position), out [T, heads, kv_rank] = sum_j p_ij c_j -- any strides over tokens and heads.  ``q_len_range`` (shortest, longest
     segment) and ``max_kv_len`` (longest ctx_len + q_len), known on the host, choose the work split of the matrix-core kernel,
-    which serves the sizes ``latent_attention_fast_supported`` names; ``plain`` forces the fp32-math kernel of any size."""
-    _cuda(out, q_lat, q_rot, cache, block_tables, q_start, q_len, ctx_len, seq_of_token, inv_freq)
+    which serves the sizes ``latent_attention_fast_supported`` names; ``plain`` forces the fp32-math kernel of any size.
+    ``window`` > 0: a row sees only the last ``window`` keys up to its own; ``sink`` fp32 [heads]: exp(sink) joins every row's
+    softmax denominator (unscaled, without a value)."""
+    _cuda(out, q_lat, q_rot, cache, block_tables, q_start, q_len, ctx_len, seq_of_token, inv_freq, sink)
+    _need(sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == q_lat.shape[1]),
+          "latent_attention: sink fp32 [heads]")
+    window = max(int(window), 0)
     T, H, R = q_lat.shape
     nb, bs, D = cache.shape
     P_ = D - R
@@ -612,12 +618,14 @@ def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: Optional[tor
         check(lib.aphro_latent_attention_plain(
             out.data_ptr(), os_, ohs, q_lat.data_ptr(), qs, qhs, _p(q_rot), rs, rhs, cache.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], nb, bs, q_start.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), _p(inv_freq), float(mscale),
-            T, H, R, P_, int(rot_dims), float(scale), _dt(q_lat), _stream()), "latent_attention")
+            T, H, R, P_, int(rot_dims), float(scale), window, _p(sink), _dt(q_lat), _stream()), "latent_attention")
         return
     lo, hi = int(q_len_range[0]), int(q_len_range[1])
     _need(0 < lo <= hi, "latent_attention: q_len_range (shortest, longest)")
     ws, ws_n = None, 0
     if lib.aphro_latent_attention_fast_supported(R, P_, int(rot_dims), _dt(q_lat)):
+        if window > 0:                         # what a row can see, not how long its sequence is, decides the split
+            max_kv_len = min(int(max_kv_len), window + hi)
         splits = int(lib.aphro_latent_attention_splits(T, S, hi, H, int(max_kv_len)))
         if splits > 1:
             ws_n = T * H * splits * (2 + R)
@@ -625,8 +633,8 @@ def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: Optional[tor
     check(lib.aphro_latent_attention(
         out.data_ptr(), os_, ohs, q_lat.data_ptr(), qs, qhs, _p(q_rot), rs, rhs, cache.data_ptr(), block_tables.data_ptr(),
         block_tables.shape[1], nb, bs, q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), _p(inv_freq),
-        float(mscale), T, S, hi, int(max_kv_len), H, R, P_, int(rot_dims), float(scale), _p(ws), ws_n, _dt(q_lat), _stream()),
-        "latent_attention")
+        float(mscale), T, S, hi, int(max_kv_len), H, R, P_, int(rot_dims), float(scale), window, _p(sink), _p(ws), ws_n, _dt(q_lat),
+        _stream()), "latent_attention")
 
 
 def latent_attention_fast_supported(kv_rank: int, rot_dim: int, rot_dims: int, dtype: torch.dtype) -> bool:
@@ -659,3 +667,158 @@ def experts_route_grouped(router_out: torch.Tensor, top: int, groups: int, keep:
     check(_lib.mixers_lib().aphro_experts_route_grouped(ids.data_ptr(), w.data_ptr(), router_out.data_ptr(), T, E, int(top), int(groups),
                                                         int(keep), int(group_top), float(scale), _stream()), "experts_route_grouped")
     return ids, w
+
+
+def experts_route_topk(router_out: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """router_out fp32 [T, experts] (+ bias fp32 [experts]) -> (ids int32 [T, top], weights fp32 [T, top]): the ``top`` largest
+    logits are chosen (ties to the lower index), the weights are the softmax over the chosen logits only."""
+    _cuda(router_out, bias)
+    T, E = router_out.shape
+    _need(router_out.dtype == torch.float32 and router_out.is_contiguous(), "experts_route_topk: router outputs fp32, contiguous")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == E and bias.is_contiguous()), "experts_route_topk: bias fp32 [experts]")
+    ids = torch.empty(T, top, dtype=torch.int32, device=router_out.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=router_out.device)
+    check(_lib.mixers_lib().aphro_experts_route_topk(ids.data_ptr(), w.data_ptr(), router_out.data_ptr(), _p(bias), T, E, int(top),
+                                                     _stream()), "experts_route_topk")
+    return ids, w
+
+
+# ---- a residual in several streams, the gated delta rule, rotary attention's preparation ---------------------------------------
+def _host_floats(values, n: int, what: str):
+    """A ctypes float array (host memory) of n numbers, or None."""
+    import ctypes
+    if values is None:
+        return None
+    vals = [float(v) for v in values]
+    _need(len(vals) == n, f"{what}: {n} numbers expected, {len(vals)} given")
+    return (ctypes.c_float * n)(*vals)
+
+
+def hyper_residual_rms_norm(x: torch.Tensor, y: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None, mix=None,
+                            out_coef=None, mult: float = 1.0, in_coef=None, weight: Optional[torch.Tensor] = None,
+                            eps: float = 1e-6, dtype: Optional[torch.dtype] = None, want_out: bool = True,
+                            want_sum: bool = False):
+    """x fp32 [T, streams, W] in place.  With ``y`` [T, W]: every stream t becomes sum_s mix[s][t] x_s + mult * out_coef[t] *
+    (scale * y).  Then u = sum_s in_coef[s] x_s and the result is rms_norm(u) * weight in the activation dtype (``want_out``
+    False: none); ``want_sum``: u itself (fp32 [T, W]) is returned as a second value.  mix (rows of [from][to]), out_coef and
+    in_coef are host numbers (None: identity / ones); scale and weight are [W] tensors of the activation dtype (None: ones)."""
+    import ctypes
+    _cuda(x, y, scale, weight)
+    _need(x.dim() == 3 and x.dtype == torch.float32 and x.is_contiguous(), "hyper_residual_rms_norm: x fp32 [T, streams, W], contiguous")
+    T, n, W = x.shape
+    some = next((t for t in (y, weight, scale) if t is not None), None)
+    adt = dtype or (some.dtype if some is not None else None)
+    _need(adt in _DT, "hyper_residual_rms_norm: the activation dtype is not given")
+    ys = 0
+    if y is not None:
+        _need(y.dtype == adt and y.shape[0] == T, "hyper_residual_rms_norm: y [T, W] of the activation dtype")
+        ys = _rows(y, W, "hyper_residual_rms_norm y")
+    for v in (scale, weight):
+        _need(v is None or (v.dtype == adt and v.numel() == W and v.is_contiguous()), "hyper_residual_rms_norm: vectors [W] of the activation dtype")
+    mixa = _host_floats(None if mix is None else [c for row in mix for c in row], n * n, "hyper_residual_rms_norm mix")
+    outa = _host_floats(out_coef, n, "hyper_residual_rms_norm out_coef")
+    ina = _host_floats(in_coef, n, "hyper_residual_rms_norm in_coef")
+    out = torch.empty(T, W, dtype=adt, device=x.device) if want_out else None
+    total = torch.empty(T, W, dtype=torch.float32, device=x.device) if want_sum else None
+    ptr = lambda a: None if a is None else ctypes.cast(a, ctypes.c_void_p)
+    check(_lib.mixers_lib().aphro_hyper_residual_rms_norm(x.data_ptr(), _p(y), ys, _p(scale), ptr(mixa), ptr(outa), float(mult), ptr(ina),
+                                                          _p(weight), _p(out), _p(total), T, n, W, float(eps), _DT[adt], _stream()),
+          "hyper_residual_rms_norm")
+    return (out, total) if want_sum else out
+
+
+def logit_softcap(z: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+    """fp32 ``cap * tanh(z * scale / cap)`` (``cap`` <= 0: ``z * scale``) of a contiguous tensor of the activation dtype."""
+    _cuda(z)
+    _need(z.is_contiguous(), "logit_softcap: contiguous input")
+    out = torch.empty(z.shape, dtype=torch.float32, device=z.device)
+    check(_lib.mixers_lib().aphro_logit_softcap(out.data_ptr(), z.data_ptr(), z.numel(), float(scale), float(cap), _dt(z), _stream()),
+          "logit_softcap")
+    return out
+
+
+def gated_delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b: torch.Tensor, a: torch.Tensor, a_log: torch.Tensor,
+                     dt_bias: torch.Tensor, state: torch.Tensor, slot_of_seq: torch.Tensor, q_start: torch.Tensor,
+                     q_len: torch.Tensor, ctx_len: torch.Tensor, heads: int, kv_heads: int, q_scale: float, norm_eps: float = 1e-6,
+                     max_q_len: int = 1) -> torch.Tensor:
+    """Scan every segment through its slot's state S fp32 [slots, heads, dim, vdim] (updated in place) with the gated delta rule;
+    returns o fp32 [T, heads * vdim].  q, k [T, kv_heads * dim] (made unit vectors per head inside), v [T, heads * vdim], b and a
+    [T, heads] raw (beta = sigmoid(b), decay = exp(-exp(a_log) softplus(a + dt_bias))); a_log, dt_bias fp32 [heads]."""
+    _cuda(q, k, v, b, a, a_log, dt_bias, state, slot_of_seq, q_start, q_len, ctx_len)
+    T, S = q.shape[0], q_start.numel()
+    _need(state.dim() == 4 and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == heads,
+          "gated_delta_scan: state fp32 [slots, heads, dim, vdim]")
+    slots, _, d, e = state.shape
+    _need(q.dtype == k.dtype == v.dtype == b.dtype == a.dtype and k.shape[0] == T and v.shape[0] == T and b.shape[0] == T
+          and a.shape[0] == T, "gated_delta_scan: q, k, v, b, a rows / dtype")
+    for t, nm in ((a_log, "a_log"), (dt_bias, "dt_bias")):
+        _need(t.dtype == torch.float32 and t.numel() == heads and t.is_contiguous(), f"gated_delta_scan: {nm} fp32 [heads]")
+    for t, nm in ((slot_of_seq, "slot_of_seq"), (q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+        _i32(t, S, nm)
+    out = torch.empty(T, heads * e, dtype=torch.float32, device=q.device)
+    check(_lib.mixers_lib().aphro_gated_delta_scan(
+        out.data_ptr(), q.data_ptr(), _rows(q, kv_heads * d, "q"), k.data_ptr(), _rows(k, kv_heads * d, "k"), v.data_ptr(),
+        _rows(v, heads * e, "v"), b.data_ptr(), _rows(b, heads, "b"), a.data_ptr(), _rows(a, heads, "a"), a_log.data_ptr(),
+        dt_bias.data_ptr(), state.data_ptr(), slot_of_seq.data_ptr(), slots, q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
+        S, T, heads, kv_heads, d, e, float(q_scale), float(norm_eps), int(max_q_len), _dt(q), _stream()), "gated_delta_scan")
+    return out
+
+
+GATE_SIGMOID, GATE_SILU = 0, 1
+
+
+def gated_head_rms_norm(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor], gate: Optional[torch.Tensor],
+                        heads: int, eps: float, act: int = GATE_SIGMOID) -> None:
+    """out [T, heads * vdim] (dense rows, any row stride) = x / rms(x over each head) * weight[vdim] * act(gate); x fp32
+    [T, heads * vdim] contiguous; weight is shared by the heads."""
+    _cuda(out, x, weight, gate)
+    T, N = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and N % heads == 0, "gated_head_rms_norm: x fp32 [T, heads * vdim], contiguous")
+    e = N // heads
+    _need(out.shape == (T, N), "gated_head_rms_norm: out [T, heads * vdim]")
+    _need(weight is None or (weight.dtype == out.dtype and weight.numel() == e and weight.is_contiguous()), "gated_head_rms_norm: weight [vdim]")
+    gs = 0
+    if gate is not None:
+        _need(gate.dtype == out.dtype and gate.shape == (T, N), "gated_head_rms_norm: gate [T, heads * vdim] of the output dtype")
+        gs = _rows(gate, N, "gated_head_rms_norm gate")
+    check(_lib.mixers_lib().aphro_gated_head_rms_norm(out.data_ptr(), _rows(out, N, "gated_head_rms_norm out"), x.data_ptr(), _p(weight),
+                                                      _p(gate), gs, T, heads, e, float(eps), int(act), _dt(out), _stream()),
+          "gated_head_rms_norm")
+
+
+ROTARY_HALF, ROTARY_INTERLEAVED = 0, 1
+
+
+def rotary_qk_norm_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                            slot_mapping: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor, seq_of_token: torch.Tensor,
+                            inv_freq: Optional[torch.Tensor], rot_dims: int, layout: int = ROTARY_HALF, qk_norm: bool = False,
+                            eps: float = 1e-6, v_other: Optional[torch.Tensor] = None, lam: float = 0.0) -> torch.Tensor:
+    """q [T, heads * dim], k [T, kv_heads * dim], v [T, kv_heads * vdim] (dense rows of one input product): rotates the first
+    ``rot_dims`` numbers of every q and k head at the row's position, optionally brings every q and k head to unit RMS, blends v
+    with ``v_other`` ((1 - lam) v + lam v_other), writes k and v into the paged caches k_cache [blocks, block, kv_heads, dim] /
+    v_cache [.., vdim] at ``slot_mapping`` and returns the prepared queries [T, heads * dim]."""
+    _cuda(q, k, v, k_cache, v_cache, slot_mapping, q_start, ctx_len, seq_of_token, inv_freq, v_other)
+    nb, bs, G, d = k_cache.shape
+    e = v_cache.shape[3]
+    T, S = q.shape[0], q_start.numel()
+    _need(v_cache.shape[:3] == (nb, bs, G) and k_cache.is_contiguous() and v_cache.is_contiguous(), "rotary_qk_norm_kv_write: cache shapes")
+    _need(q.dim() == 2 and q.shape[1] % d == 0 and k.shape[0] == T and v.shape[0] == T, "rotary_qk_norm_kv_write: q [T, heads * dim]")
+    H = q.shape[1] // d
+    _need(q.dtype == k.dtype == v.dtype == k_cache.dtype == v_cache.dtype, "rotary_qk_norm_kv_write: one dtype")
+    _need(slot_mapping.dtype == torch.int64 and slot_mapping.numel() == T and slot_mapping.is_contiguous(), "rotary_qk_norm_kv_write: slots int64 [T]")
+    _i32(q_start, S, "q_start")
+    _i32(ctx_len, S, "ctx_len")
+    _i32(seq_of_token, T, "seq_of_token")
+    _need(rot_dims == 0 or (inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2
+                            and inv_freq.is_contiguous()), "rotary_qk_norm_kv_write: inv_freq fp32 [rot_dims / 2]")
+    vos = 0
+    if v_other is not None:
+        _need(v_other.dtype == v.dtype and v_other.shape[0] == T, "rotary_qk_norm_kv_write: v_other [T, kv_heads * vdim]")
+        vos = _rows(v_other, G * e, "v_other")
+    q_out = torch.empty(T, H * d, dtype=q.dtype, device=q.device)
+    check(_lib.mixers_lib().aphro_rotary_qk_norm_kv_write(
+        q_out.data_ptr(), H * d, k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), nb * bs, q.data_ptr(),
+        _rows(q, H * d, "q"), k.data_ptr(), _rows(k, G * d, "k"), v.data_ptr(), _rows(v, G * e, "v"), _p(v_other), vos, float(lam),
+        q_start.data_ptr(), ctx_len.data_ptr(), seq_of_token.data_ptr(), _p(inv_freq), T, H, G, d, e, int(rot_dims), int(layout),
+        1 if qk_norm else 0, float(eps), _dt(q), _stream()), "rotary_qk_norm_kv_write")
+    return q_out

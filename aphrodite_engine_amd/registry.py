@@ -60,8 +60,13 @@ def _register_builtin() -> None:
         from .fekotar import load_fekotar
         return load_fekotar(model_dir, config, **kw)
 
+    def pagulix(model_dir, config, **kw):
+        from .pagulix import load_pagulix
+        return load_pagulix(model_dir, config, **kw)
+
     for arch in ("LlamaForCausalLM", "MistralForCausalLM", "MixtralForCausalLM"):
         _LOADERS.setdefault(arch, llama)
     _LOADERS.setdefault("Fatudra", fatudra)
     _LOADERS.setdefault("Gipozen", gipozen)
     _LOADERS.setdefault("Fekotar", fekotar)
+    _LOADERS.setdefault("Pagulix", pagulix)

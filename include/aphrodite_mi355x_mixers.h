@@ -129,12 +129,12 @@ int aphro_differential_norm_gate(void* out, int64_t out_stride, const float* a, 
  * k_cache [cache slots, ck] / v_cache [cache slots, cv] at row cache_slots[t] (int64; outside 0 .. num_cache_slots - 1: skipped).
  * ck == cv == 0: no cache.  state [state slots, taps - 1, channels] of `dtype` holds each request's last taps - 1 inputs:
  * read for the rows before a segment (never for positions before the sequence's start), rewritten afterwards.
- * 1 <= taps <= 16. */
+ * 1 <= taps <= 16.  act: 0 none, 1 silu on the convolution's result. */
 int aphro_short_conv(void* q_out, int64_t q_out_stride, void* k_cache, void* v_cache, const int64_t* cache_slots,
                      int64_t num_cache_slots, const void* u, int64_t u_stride, const void* w, void* state,
                      const int32_t* state_slots, const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
-                     const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int cq, int ck, int cv, int taps, int dtype,
-                     void* stream);
+                     const int32_t* seq_of_token, int64_t num_tokens, int num_seqs, int cq, int ck, int cv, int taps, int act,
+                     int dtype, void* stream);
 
 /* Softmax attention under a sliding window that keeps the first tokens: row i sees key j if j <= i and
  * (i - j < window or j < keep_first); window <= 0: every earlier key.  No rotation, no bias.  A head carries `maps`
@@ -228,13 +228,15 @@ int aphro_latent_prep(void* cq, void* cache, int64_t num_cache_rows, const void*
                       int rot_dim, int rot_dims, float eps, int dtype, void* stream);
 /* Causal softmax attention of every head over the shared latent rows cache [blocks, block, kv_rank + rot_dim]:
  * score = ([q_lat | rotate(q_rot)] . row) * scale, out = sum p * row[:kv_rank].  q_lat / q_rot / out are addressed as
- * base + t * stride + head * head_stride (elements); any sizes (kv_rank <= 1024), fp32 math. */
+ * base + t * stride + head * head_stride (elements); any sizes (kv_rank <= 1024), fp32 math.
+ * window > 0: row i sees key j only if i - j < window.  sink fp32 [heads] (NULL: none): exp(sink[head]) -- not scaled -- is
+ * one more term of the softmax denominator, without a value. */
 int aphro_latent_attention_plain(void* out, int64_t out_stride, int64_t out_head_stride, const void* q_lat, int64_t ql_stride,
                                  int64_t ql_head_stride, const void* q_rot, int64_t qr_stride, int64_t qr_head_stride,
                                  const void* cache, const int32_t* block_tables, int max_blocks, int64_t num_blocks, int block_size,
                                  const int32_t* q_start, const int32_t* ctx_len, const int32_t* seq_of_token, const float* inv_freq,
                                  float mscale, int64_t num_tokens, int heads, int kv_rank, int rot_dim, int rot_dims, float scale,
-                                 int dtype, void* stream);
+                                 int window, const float* sink, int dtype, void* stream);
 /* The same attention with the kernel chosen by size: bf16 with (kv_rank, rot_dim) in {(128, 16), (128, 32), (256, 32), (256, 64),
  * (512, 64)}, rot_dims == rot_dim and 16-byte aligned rows run on the matrix cores (aphro_latent_attention_fast_supported), the
  * query rows of a segment flattened to (token, head) pairs, 64 per workgroup; everything else runs the kernel above.  min/max
@@ -247,8 +249,8 @@ int aphro_latent_attention(void* out, int64_t out_stride, int64_t out_head_strid
                            const int32_t* block_tables, int max_blocks, int64_t num_blocks, int block_size, const int32_t* q_start,
                            const int32_t* q_len, const int32_t* ctx_len, const int32_t* seq_of_token, const float* inv_freq,
                            float mscale, int64_t num_tokens, int num_seqs, int max_q_len, int max_kv_len, int heads, int kv_rank,
-                           int rot_dim, int rot_dims, float scale, float* workspace, int64_t workspace_floats, int dtype,
-                           void* stream);
+                           int rot_dim, int rot_dims, float scale, int window, const float* sink, float* workspace,
+                           int64_t workspace_floats, int dtype, void* stream);
 /* out[t, i] = x[t, i] * sigmoid(gate[t, i]), i < n (out may be x) */
 int aphro_sigmoid_gate_mul(void* out, int64_t out_stride, const void* x, int64_t x_stride, const void* gate, int64_t gate_stride,
                            int64_t num_tokens, int n, int dtype, void* stream);
@@ -257,6 +259,56 @@ int aphro_sigmoid_gate_mul(void* out, int64_t out_stride, const void* x, int64_t
  * int32 [T, top] are the `top` largest s among them, weights fp32 [T, top] = s * scale. */
 int aphro_experts_route_grouped(int32_t* ids, float* weights, const float* router_out, int64_t num_tokens, int experts, int top,
                                 int groups, int keep, int group_top, float scale, void* stream);
+
+/* Router whose weights are the softmax over the chosen logits only: the `top` largest of router_out + bias (fp32 [outputs],
+ * NULL: none; ties to the lower index) are chosen, weights = softmax over those `top` logits. */
+int aphro_experts_route_topk(int32_t* ids, float* weights, const float* router_out, const float* bias, int64_t num_tokens,
+                             int outputs, int top, void* stream);
+
+/* ---- a residual in several streams, the gated delta rule, rotary attention's preparation ------------------------------------ */
+
+/* Hyper-connections around x fp32 [T, streams, width], both halves optional:
+ *   write (y != NULL):  x_t <- sum_s mix[s, t] x_s + mult * out_coef[t] * (scale (.) y)   all streams from the old ones
+ *   read (out != NULL): u = sum_s in_coef[s] x_s;  out = u / sqrt(mean(u^2) + eps) * weight;  sum_out (fp32 [T, width], NULL: not
+ *                       written) = u
+ * y [T, width] (row stride), scale and weight [width] of `dtype` (NULL: ones); mix [streams, streams] indexed [from, to] (NULL:
+ * identity), out_coef and in_coef [streams] (NULL: ones) are HOST arrays of floats, copied into the launch.  streams <= 16. */
+int aphro_hyper_residual_rms_norm(float* x, const void* y, int64_t y_stride, const void* scale, const float* mix,
+                                  const float* out_coef, float mult, const float* in_coef, const void* weight, void* out,
+                                  float* sum_out, int64_t num_tokens, int streams, int width, float eps, int dtype, void* stream);
+/* out[i] = cap * tanh(in[i] * scale / cap)  (cap <= 0: in[i] * scale); in of `dtype`, out fp32, n numbers */
+int aphro_logit_softcap(float* out, const void* in, int64_t n, float scale, float cap, int dtype, void* stream);
+
+/* Gated delta rule, one state S fp32 [dim, vdim] per (slot, head):
+ *   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q      (the read-out sees the current token's write)
+ * q, k [T, kv_heads * dim] are made unit vectors per head here (x / sqrt(sum x^2 + norm_eps); q times q_scale); value head h
+ * uses query / key head h / (heads / kv_heads); v [T, heads * vdim]; beta = sigmoid(b), g = exp(-exp(a_log[h]) *
+ * softplus(a + dt_bias[h])) from b, a [T, heads] (row strides, `dtype`); a_log, dt_bias fp32 [heads].  out fp32 [T, heads * vdim].
+ * state fp32 [slots, heads, dim, vdim]; a segment with ctx_len == 0 starts from zero without reading its slot.  dim <= 256.
+ * max_q_len (host: longest segment) picks the work split. */
+int aphro_gated_delta_scan(float* out, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                           int64_t v_stride, const void* b, int64_t b_stride, const void* a, int64_t a_stride, const float* a_log,
+                           const float* dt_bias, float* state, const int32_t* slot_of_seq, int num_slots, const int32_t* q_start,
+                           const int32_t* q_len, const int32_t* ctx_len, int num_seqs, int64_t num_tokens, int heads, int kv_heads,
+                           int dim, int vdim, float q_scale, float norm_eps, int max_q_len, int dtype, void* stream);
+/* out[t, h, i] = x[t, h, i] / sqrt(mean_i x^2 + eps) * weight[i] * act(gate[t, h, i]); x fp32 [T, heads * vdim] contiguous;
+ * weight [vdim] (shared by the heads; NULL: ones), gate (row stride; NULL: none) and out (row stride) of `dtype`;
+ * act 0: sigmoid, 1: silu. */
+int aphro_gated_head_rms_norm(void* out, int64_t out_stride, const float* x, const void* weight, const void* gate,
+                              int64_t gate_stride, int64_t num_tokens, int heads, int vdim, float eps, int act, int dtype,
+                              void* stream);
+
+/* From the rows of a rotary attention's input product: the first rot_dims numbers of every query and key head turned by
+ * position * inv_freq[i] (layout 0: number i pairs with i + rot_dims / 2; 1: number 2 i with 2 i + 1), then -- qk_norm != 0 --
+ * every query and key head divided by sqrt(mean(x^2) + eps); values blended v <- (1 - lambda) v + lambda v_other (v_other NULL:
+ * none).  Queries go to q_out [T, heads * dim], keys and values into k_cache [rows, kv_heads, dim] / v_cache [rows, kv_heads,
+ * vdim] at slot_mapping[t] (outside 0 .. num_cache_rows - 1: skipped).  dim <= 512. */
+int aphro_rotary_qk_norm_kv_write(void* q_out, int64_t q_out_stride, void* k_cache, void* v_cache, const int64_t* slot_mapping,
+                                  int64_t num_cache_rows, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
+                                  const void* v, int64_t v_stride, const void* v_other, int64_t v_other_stride, float lambda,
+                                  const int32_t* q_start, const int32_t* ctx_len, const int32_t* seq_of_token, const float* inv_freq,
+                                  int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int rot_dims, int layout,
+                                  int qk_norm, float eps, int dtype, void* stream);
 
 #ifdef __cplusplus
 }
