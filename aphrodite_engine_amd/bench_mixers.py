@@ -1,4 +1,4 @@
-"""``bench.py --mixers [--mixers-design fatudra|gipozen|fekotar]``: prefill and decode throughput of a Fatudra (or Gipozen) stack at sizes that resemble a real model's layers
+"""``bench.py --mixers [--mixers-design fatudra|gipozen|fekotar|pagulix]``: prefill and decode throughput of a Fatudra (or Gipozen) stack at sizes that resemble a real model's layers
 (random bf16 weights), beside a Llama stack of equal width / heads / feed-forward / layer count on the unquantised op path,
 plus each mixer kernel alone against its roofline and against the like kernel of the Llama path.  Prints ONE JSON line;
 the default workload of bench.py is untouched by it.  The Gipozen stack: windowed differential attention (two maps of half the
@@ -10,6 +10,11 @@ The Fekotar stack: attention through a cached latent of rank 512 + 64 rotated nu
 width), heads of 128 + 64 / 128, a dense clamped feed-forward in the first layer and 16 silu experts (top 4 of the 2 best of 4
 groups, a quarter of the dense feed-forward each) in the others; it stands beside Llama AND beside the Gipozen stack (the
 closest existing model: its own attention kernels plus routed experts) at equal width.
+
+The Pagulix stack: a gated-delta layer (16 / 32 value heads of 128 x 128 state over 4 / 8 query-key heads, 4-tap convolutions), a
+latent attention layer (rank 512 + 64 rotated numbers, window 1024, sinks), two rotary attention layers with unit-RMS q / k and
+blended values, four residual streams, 16 silu experts (top 4, softmax over the chosen) plus a shared expert in every layer; it
+stands beside the Fekotar stack (the closest existing model) and Llama.
 
 Rooflines used: 8 TB/s HBM for the memory-bound kernels (norms, activations, decode attention, the decode step of the
 memories: their state is read and written once), 2.5 PFLOP/s dense bf16 MFMA for prompt attention (4 d flops per visible
@@ -451,8 +456,203 @@ def fekotar_kernel_section(s, prompt_len, batch, ctx, device):
     return out
 
 
+PAG_RANK, PAG_ROT, PAG_WINDOW, PAG_EXPERTS, PAG_TOP, PAG_STREAMS, PAG_TAPS = 512, 64, 1024, 16, 4, 4, 4
+
+
+def pagulix_config(s):
+    """delta, windowed latent attention, two rotary attentions that blend values; four streams; 16 experts (top 4) + a shared one"""
+    eff = s["ff"] // 4 // 32 * 32
+    moe = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": PAG_EXPERTS, "top": PAG_TOP}, "shared": {"ff": eff}}
+    rot = {"base": 500000.0, "dims": s["dim"] // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    delta = {"type": "delta", "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "conv": PAG_TAPS}}
+    latent = {"type": "latent_attention",
+              "mixer": {"heads": s["heads"], "dim": s["dim"], "rot_dim": PAG_ROT, "vdim": s["dim"], "kv_rank": PAG_RANK,
+                        "scale": (s["dim"] + PAG_ROT) ** -0.5, "mask": {"size": PAG_WINDOW}, "rot": {"base": 10000.0, "dims": PAG_ROT}}}
+    attn = {"type": "attention", "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "rot": rot,
+                                           "scale": s["dim"] ** -0.5, "v_mix": True}}
+    layers = [dict(l, mlp=moe) for l in (delta, latent, attn, attn)][:LAYERS]
+    return {"architecture": "Pagulix", "vocab": VOCAB, "width": s["width"], "norm": {"eps": 1e-6}, "streams": PAG_STREAMS,
+            "residual_mult": 0.3, "logit_softcap": 30.0, "layers": layers}
+
+
+def pagulix_kernel_section(s, prompt_len, batch, ctx, device):
+    """Each kernel that Pagulix adds (or extends) alone at the stack's shapes, beside the like kernel of the closest existing path."""
+    from . import _custom_ops as ops
+    from . import mixer_ops as mops
+    from .mixers import LatentCacheSpec, RotaryFrequencies
+    bf = torch.bfloat16
+    H, G, d, W, ff = s["heads"], s["kv_heads"], s["dim"], s["width"], s["ff"]
+    R, P, n = PAG_RANK, PAG_ROT, PAG_STREAMS
+    pre, dec, pages = batches(prompt_len, batch, ctx, device, VOCAB)
+    out = {}
+
+    def rec(name, sec, bytes_=None, flops=None, like=None):
+        r = {"us": round(sec * 1e6, 1)}
+        if bytes_ is not None:
+            r["frac_hbm"] = round(bytes_ / sec / HBM, 3)
+        if flops is not None:
+            r["frac_mfma"] = round(flops / sec / MFMA, 4)
+        if like is not None:
+            r["like"] = like
+        out[name] = r
+
+    rot = RotaryFrequencies(P, 10000.0).to(device)
+    rot_a = RotaryFrequencies.wavelength_scaled(d // 2, 500000.0, 8.0, 1.0, 4.0, 8192).to(device)
+    cache = LatentCacheSpec(R, P).allocate(pages, BLOCK, batch, bf, device)
+    cache.normal_()
+    sink = torch.randn(H, device=device)
+    kc = torch.randn(pages, BLOCK, G, d, device=device, dtype=bf)
+    vc = torch.randn(pages, BLOCK, G, d, device=device, dtype=bf)
+    for name, b, T in (("prefill", pre, prompt_len), ("decode", dec, batch)):
+        lens = (min(b.q_lens), max(b.q_lens))
+        kvmax = max(c + q for c, q in zip(b.ctx_lens, b.q_lens))
+        # ---- the streamed residual: write of one sublayer + read and norm of the next -------------------------------------------
+        x = torch.randn(T, n, W, device=device)
+        y, ls, w16 = torch.randn(T, W, device=device, dtype=bf), torch.randn(W, device=device, dtype=bf), torch.randn(W, device=device, dtype=bf)
+        mix = (torch.eye(n) + 0.1 * torch.randn(n, n)).tolist()
+        oc, ic = [1.0] * n, [0.5] * n
+        sec = timed(lambda: mops.hyper_residual_rms_norm(x, y, ls, mix, oc, 0.3, ic, w16, 1e-6))
+        x16, r16 = torch.randn(T, W, device=device, dtype=bf), torch.randn(T, W, device=device, dtype=bf)
+        lsec = timed(lambda: ops.fused_add_rms_norm(x16, r16, w16, 1e-5))
+        rec("hyper_residual_rms_norm_" + name, sec, bytes_=T * W * (8 * n + 4),
+            like={"kernel": "fused_add_rms_norm", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * W * 8 / lsec / HBM, 3)})
+        # ---- the gated delta rule beside the decay memory of equal shape ------------------------------------------------------------
+        q, k = torch.randn(T, G * d, device=device, dtype=bf), torch.randn(T, G * d, device=device, dtype=bf)
+        v = torch.randn(T, H * d, device=device, dtype=bf)
+        bb, aa = torch.randn(T, H, device=device, dtype=bf), torch.randn(T, H, device=device, dtype=bf)
+        a_log, dtb = torch.zeros(H, device=device), torch.zeros(H, device=device)
+        state = torch.zeros(batch, H, d, d, device=device)
+        sec = timed(lambda: mops.gated_delta_scan(q, k, v, bb, aa, a_log, dtb, state, b.state_slots, b.q_start, b.q_len, b.ctx_len, H, G,
+                                                  d ** -0.5, 1e-6, max_q_len=lens[1]))
+        qh = torch.randn(T, H * d, device=device, dtype=bf)
+        decay = torch.full((H, ), 0.97, device=device)
+        lsec = timed(lambda: mops.outer_memory_scan(qh, qh, v, (state, ), b.state_slots, b.q_start, b.q_len, b.ctx_len, H, mops.MEMORY_DECAY,
+                                                    decay, max_q_len=lens[1]))
+        like = {"kernel": "outer_memory_scan (decay)", "us": round(lsec * 1e6, 1)}
+        if name == "prefill":
+            rec("gated_delta_scan_" + name, sec, flops=T * H * 4.0 * d * d, like=dict(like, frac_mfma=round(T * H * 4.0 * d * d / lsec / MFMA, 5)))
+        else:
+            nb = batch * H * d * d * 8
+            rec("gated_delta_scan_" + name, sec, bytes_=nb, like=dict(like, frac_hbm=round(nb / lsec / HBM, 3)))
+        o32, gate, wn = torch.randn(T, H * d, device=device), torch.randn(T, H * d, device=device, dtype=bf), torch.randn(d, device=device, dtype=bf)
+        yo = torch.empty(T, H * d, device=device, dtype=bf)
+        sec = timed(lambda: mops.gated_head_rms_norm(yo, o32, wn, gate, H, 1e-6, mops.GATE_SILU))
+        wfull = wn.repeat(H)
+        lsec = timed(lambda: mops.gated_group_rms_norm(yo, o32, wfull, gate, d, 1e-6))
+        rec("gated_head_rms_norm_" + name, sec, bytes_=T * H * d * 8,
+            like={"kernel": "gated_group_rms_norm", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * H * d * 8 / lsec / HBM, 3)})
+        C = 2 * G * d + H * d
+        u, cw = torch.randn(T, C, device=device, dtype=bf), torch.randn(C, PAG_TAPS, device=device, dtype=bf)
+        cstate = torch.zeros(batch, PAG_TAPS - 1, C, device=device, dtype=bf)
+        sec = timed(lambda: mops.short_conv(u, cw, cstate, b.state_slots, b.q_start, b.q_len, b.ctx_len, b.seq_of_token, C, act=1))
+        lsec = timed(lambda: mops.short_conv(u, cw, cstate, b.state_slots, b.q_start, b.q_len, b.ctx_len, b.seq_of_token, C))
+        rec("short_conv_silu_" + name, sec, bytes_=T * C * 4,
+            like={"kernel": "short_conv (no activation)", "us": round(lsec * 1e6, 1), "frac_hbm": round(T * C * 4 / lsec / HBM, 3)})
+        # ---- rotation + unit RMS + value blend + cache write ---------------------------------------------------------------------------
+        pq, pk, pv = torch.randn(T, H * d, device=device, dtype=bf), torch.randn(T, G * d, device=device, dtype=bf), torch.randn(T, G * d, device=device, dtype=bf)
+        vo = torch.randn(T, G * d, device=device, dtype=bf)
+        sec = timed(lambda: mops.rotary_qk_norm_kv_write(pq, pk, pv, kc, vc, b.slot_mapping, b.q_start, b.ctx_len, b.seq_of_token,
+                                                         rot_a.inv_freq, d // 2, mops.ROTARY_HALF, True, 1e-6, vo, 0.3))
+        lkc = torch.zeros(pages, G, d // 8, BLOCK, 8, device=device, dtype=bf)
+        lvc = torch.zeros(pages, G, d, BLOCK, device=device, dtype=bf)
+        cs = torch.randn(8192, d, device=device, dtype=bf)
+        k3 = pk.view(T, G, d)
+        lsec = timed(lambda: (ops.rotary_embedding(b.positions, pq, pk, d, cs, True),
+                              ops.reshape_and_cache(k3, k3, lkc, lvc, b.slot_mapping, "auto", 1.0, 1.0)))
+        rec("rotary_qk_norm_kv_write_" + name, sec, bytes_=T * ((2 * H + 5 * G) * d) * 2,
+            like={"kernel": "rotary_embedding + reshape_and_cache", "us": round(lsec * 1e6, 1),
+                  "frac_hbm": round(T * (H + 3 * G) * d * 4 / lsec / HBM, 3)})
+        # ---- causal attention on the kernels of the distance-biased attention, no bias ----------------------------------------------------
+        o = torch.empty(T, H * d, device=device, dtype=bf)
+        sec = timed(lambda: mops.distance_bias_attention(o, pq, None, kc, vc, b.block_tables, b.q_start, b.q_len, b.ctx_len, b.seq_of_token,
+                                                         lens, H, d ** -0.5, None, max_kv_len=kvmax))
+        lq = pq.view(T, H, d)
+        if name == "prefill":
+            pairs = T * (T + 1) / 2
+            kk, vv = torch.randn(T, G, d, device=device, dtype=bf), torch.randn(T, G, d, device=device, dtype=bf)
+            cu = torch.tensor([0, T], dtype=torch.int32, device=device)
+            lsec = timed(lambda: ops.flash_attn_varlen(lq, kk, vv, cu, T, d ** -0.5, causal=True))
+            rec("attention_prefill", sec, flops=pairs * H * 4.0 * d,
+                like={"kernel": "flash_attn_varlen", "us": round(lsec * 1e6, 1), "frac_mfma": round(pairs * H * 4.0 * d / lsec / MFMA, 4)})
+        else:
+            lens_t = torch.full((batch, ), ctx + 1, dtype=torch.int32, device=device)
+            lo = torch.empty(T, H, d, device=device, dtype=bf)
+            lsec = timed(lambda: ops.paged_attention_v1(lo, lq, lkc, lvc, G, d ** -0.5, b.block_tables, lens_t, BLOCK, ctx + 1, None, "auto", 1.0, 1.0))
+            nb = batch * (ctx + 1) * G * 2 * d * 2
+            rec("attention_decode", sec, bytes_=nb, like={"kernel": "paged_attention_v1", "us": round(lsec * 1e6, 1), "frac_hbm": round(nb / lsec / HBM, 3)})
+        # ---- attention in the latent under a window, with a sink -- beside the same launch without either ------------------------------
+        q_lat = torch.randn(T, H, R, device=device, dtype=bf) * R ** -0.5
+        qr = torch.randn(T, H, P, device=device, dtype=bf)
+        ol = torch.empty(T, H, R, device=device, dtype=bf)
+        la = lambda w, sk: mops.latent_attention(ol, q_lat, qr, cache, b.block_tables, b.q_start, b.q_len, b.ctx_len, b.seq_of_token, lens,
+                                                 rot.inv_freq, 1.0, P, (d + P) ** -0.5, max_kv_len=kvmax, window=w, sink=sk)
+        sec = timed(lambda: la(PAG_WINDOW, sink))
+        lsec = timed(lambda: la(0, None))
+        if name == "prefill":
+            wpairs = sum(min(i + 1, PAG_WINDOW) for i in range(T))
+            per = H * (2.0 * (R + P) + 2.0 * R)
+            rec("latent_attention_window_prefill", sec, flops=wpairs * per,
+                like={"kernel": "latent attention, causal, no sink", "us": round(lsec * 1e6, 1),
+                      "frac_mfma": round(T * (T + 1) / 2 * per / lsec / MFMA, 4)})
+        else:
+            rec("latent_attention_window_decode", sec, bytes_=batch * min(ctx + 1, PAG_WINDOW) * (R + P) * 2,
+                like={"kernel": "latent attention, causal, no sink", "us": round(lsec * 1e6, 1),
+                      "frac_hbm": round(batch * (ctx + 1) * (R + P) * 2 / lsec / HBM, 3)})
+        # ---- router ----------------------------------------------------------------------------------------------------------------------
+        zr, rb = torch.randn(T, PAG_EXPERTS, device=device), torch.randn(PAG_EXPERTS, device=device)
+        sec = timed(lambda: mops.experts_route_topk(zr, rb, PAG_TOP))
+        lsec = timed(lambda: mops.experts_route_grouped(zr, PAG_TOP, 4, 2, 1.0))
+        rec("experts_route_topk_" + name, sec, like={"kernel": "experts_route_grouped", "us": round(lsec * 1e6, 1)})
+    z = torch.randn(batch, VOCAB, device=device, dtype=bf)
+    sec = timed(lambda: mops.logit_softcap(z, 1.0, 30.0))
+    lsec = timed(lambda: z.float() * 1.0)
+    rec("logit_softcap_decode", sec, bytes_=batch * VOCAB * 6, like={"kernel": "cast and scale", "us": round(lsec * 1e6, 1),
+                                                                     "frac_hbm": round(batch * VOCAB * 6 / lsec / HBM, 3)})
+    return out
+
+
+def main_pagulix(args) -> int:
+    from . import _lib
+    from .fekotar import FekotarConfig, FekotarForCausalLM
+    from .model import LlamaConfig, LlamaForCausalLM
+    from .pagulix import PagulixConfig, PagulixForCausalLM
+    _lib.lib()
+    _lib.mixers_lib()
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    prompt_len, batch, ctx = args.mixers_prompt, args.batch, args.ctx
+    result = {"metric": "pagulix_vs_llama_bf16_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+              "n_gpus": 1, "layers": LAYERS, "sizes": {}}
+    with torch.no_grad():
+        for name, s in SIZES.items():
+            if args.mixers_size and name != args.mixers_size:
+                continue
+            t0 = time.time()
+            pag = PagulixForCausalLM(PagulixConfig.from_dict(pagulix_config(s)), torch.bfloat16).init_synthetic(device)
+            r = {"pagulix": model_throughput(pag, prompt_len, batch, ctx, device, VOCAB)}
+            del pag
+            fek = FekotarForCausalLM(FekotarConfig.from_dict(fekotar_config(s)), torch.bfloat16).init_synthetic(device)
+            r["fekotar"] = model_throughput(fek, prompt_len, batch, ctx, device, VOCAB)
+            del fek
+            lc = LlamaConfig(hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=LAYERS,
+                             num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], vocab_size=VOCAB,
+                             max_position_embeddings=max(8192, prompt_len + 16))
+            llama = LlamaForCausalLM(lc, None, torch.bfloat16).init_synthetic(device)
+            llama.use_fused_decode = False
+            r["llama"] = model_throughput(llama, prompt_len, batch, ctx, device, VOCAB)
+            del llama
+            r["kernels"] = pagulix_kernel_section(s, prompt_len, batch, ctx, device)
+            r["seconds"] = round(time.time() - t0, 1)
+            result["sizes"][name] = r
+            torch.cuda.empty_cache()
+    print(json.dumps(result), flush=True)
+    return 0
+
+
 def main(args) -> int:
     from . import _lib
+    if getattr(args, "mixers_design", "fatudra") == "pagulix":
+        return main_pagulix(args)
     if getattr(args, "mixers_design", "fatudra") == "gipozen":
         return main_gipozen(args)
     if getattr(args, "mixers_design", "fatudra") == "fekotar":

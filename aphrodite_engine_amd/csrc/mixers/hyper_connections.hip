@@ -75,6 +75,79 @@ __global__ void hyper_residual_rms_norm_kernel(float* __restrict__ x, const type
   }
 }
 
+// the same with four neighbouring channels per thread (16-byte accesses to the streams): width a multiple of 4, aligned rows
+template <typename T>
+__device__ __forceinline__ f32x4 hc_load4(const typename T::storage* p) {
+  if constexpr (sizeof(typename T::storage) == 2) {
+    const u16x4 v = *reinterpret_cast<const u16x4*>(p);
+    return f32x4{T::to_f32(v[0]), T::to_f32(v[1]), T::to_f32(v[2]), T::to_f32(v[3])};
+  } else {
+    return *reinterpret_cast<const f32x4*>(p);
+  }
+}
+template <typename T>
+__device__ __forceinline__ void hc_store4(typename T::storage* p, f32x4 v) {
+  if constexpr (sizeof(typename T::storage) == 2) {
+    *reinterpret_cast<u16x4*>(p) = u16x4{T::from_f32(v[0]), T::from_f32(v[1]), T::from_f32(v[2]), T::from_f32(v[3])};
+  } else {
+    *reinterpret_cast<f32x4*>(p) = v;
+  }
+}
+
+template <typename T, int NS>
+__global__ void hyper_residual_rms_norm_vec4_kernel(float* __restrict__ x, const typename T::storage* __restrict__ y, int64_t y_stride,
+                                                    const typename T::storage* __restrict__ scale, HCCoef cf, int has_mix,
+                                                    const typename T::storage* __restrict__ weight, typename T::storage* __restrict__ out,
+                                                    float* __restrict__ sum_out, int n, int width, float eps) {
+  extern __shared__ float u_lds[];
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  float* xr = x + t * (int64_t)n * width;
+  float ss = 0.f;
+  for (int i = 4 * threadIdx.x; i < width; i += 4 * blockDim.x) {
+    f32x4 xs[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) xs[s] = s < n ? *reinterpret_cast<const f32x4*>(xr + (int64_t)s * width + i) : f32x4{0.f, 0.f, 0.f, 0.f};
+    if (y) {
+      f32x4 yv = hc_load4<T>(y + t * y_stride + i);
+      if (scale) yv *= hc_load4<T>(scale + i);
+      f32x4 nx[NS];
+#pragma unroll
+      for (int to = 0; to < NS; ++to) {
+        f32x4 a = yv * cf.out[to];
+        if (has_mix) {
+#pragma unroll
+          for (int s = 0; s < NS; ++s)
+            if (s < n) a += xs[s] * cf.mix[s * HC_MAX_STREAMS + to];
+        } else {
+          a += xs[to];
+        }
+        nx[to] = a;
+      }
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+        if (s < n) {
+          xs[s] = nx[s];
+          *reinterpret_cast<f32x4*>(xr + (int64_t)s * width + i) = nx[s];
+        }
+    }
+    f32x4 u = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+      if (s < n) u += xs[s] * cf.in[s];
+    if (sum_out) *reinterpret_cast<f32x4*>(sum_out + t * (int64_t)width + i) = u;
+    *reinterpret_cast<f32x4*>(u_lds + i) = u;
+    ss += (u[0] * u[0] + u[1] * u[1]) + (u[2] * u[2] + u[3] * u[3]);
+  }
+  if (!out) return;
+  const float rstd = 1.0f / sqrtf(wg_sum(ss, red) / (float)width + eps);
+  for (int i = 4 * threadIdx.x; i < width; i += 4 * blockDim.x) {
+    f32x4 v = *reinterpret_cast<const f32x4*>(u_lds + i) * rstd;
+    if (weight) v *= hc_load4<T>(weight + i);
+    hc_store4<T>(out + t * (int64_t)width + i, v);
+  }
+}
+
 template <typename T>
 __global__ void logit_softcap_kernel(float* __restrict__ out, const typename T::storage* __restrict__ in, int64_t n, float scale,
                                      float cap) {
@@ -108,9 +181,19 @@ extern "C" int aphro_hyper_residual_rms_norm(float* x, const void* y, int64_t y_
   }
   const int block = width >= 1024 ? 256 : (width > 256 ? 128 : 64);
   const size_t lds = (size_t)width * sizeof(float);
+  const auto al16 = [](const void* ptr) { return ((uintptr_t)ptr & 15) == 0; };
+  const bool vec = width % 4 == 0 && y_stride % 8 == 0 && width % 8 == 0 && al16(x) && al16(y) && al16(scale) && al16(weight) && al16(out) &&
+                   al16(sum_out) && streams <= 8;
 #define HC_LAUNCH(NS)                                                                                                           \
-  hipLaunchKernelGGL((hyper_residual_rms_norm_kernel<T, NS>), dim3((unsigned)num_tokens), dim3(block), lds, (hipStream_t)stream, x, \
-                     (const S*)y, y_stride, (const S*)scale, cf, mix ? 1 : 0, (const S*)weight, (S*)out, sum_out, streams, width, eps)
+  do {                                                                                                                          \
+    if (vec)                                                                                                                    \
+      hipLaunchKernelGGL((hyper_residual_rms_norm_vec4_kernel<T, (NS > 8 ? 8 : NS)>), dim3((unsigned)num_tokens),                \
+                         dim3(width >= 1024 ? 256 : (width > 256 ? 128 : 64)), lds, (hipStream_t)stream, x, (const S*)y, y_stride, \
+                         (const S*)scale, cf, mix ? 1 : 0, (const S*)weight, (S*)out, sum_out, streams, width, eps);            \
+    else                                                                                                                        \
+      hipLaunchKernelGGL((hyper_residual_rms_norm_kernel<T, NS>), dim3((unsigned)num_tokens), dim3(block), lds, (hipStream_t)stream, x, \
+                         (const S*)y, y_stride, (const S*)scale, cf, mix ? 1 : 0, (const S*)weight, (S*)out, sum_out, streams, width, eps); \
+  } while (0)
   MIX_DISPATCH_DTYPE(dtype, {
     typedef typename T::storage S;
     if (streams == 1) HC_LAUNCH(1);

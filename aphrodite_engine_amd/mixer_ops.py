@@ -689,9 +689,20 @@ def _host_floats(values, n: int, what: str):
     import ctypes
     if values is None:
         return None
+    if isinstance(values, ctypes.Array):           # made once by the caller (host_floats)
+        _need(len(values) == n, f"{what}: {n} numbers expected, {len(values)} given")
+        return values
     vals = [float(v) for v in values]
     _need(len(vals) == n, f"{what}: {n} numbers expected, {len(vals)} given")
     return (ctypes.c_float * n)(*vals)
+
+
+def host_floats(values):
+    """A host array of floats for the coefficient arguments of ``hyper_residual_rms_norm`` (rows of a matrix are flattened), made once
+    instead of at every call."""
+    import ctypes
+    vals = [float(c) for row in values for c in (row if isinstance(row, (list, tuple)) else [row])]
+    return (ctypes.c_float * len(vals))(*vals)
 
 
 def hyper_residual_rms_norm(x: torch.Tensor, y: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None, mix=None,
@@ -715,7 +726,9 @@ def hyper_residual_rms_norm(x: torch.Tensor, y: Optional[torch.Tensor] = None, s
         ys = _rows(y, W, "hyper_residual_rms_norm y")
     for v in (scale, weight):
         _need(v is None or (v.dtype == adt and v.numel() == W and v.is_contiguous()), "hyper_residual_rms_norm: vectors [W] of the activation dtype")
-    mixa = _host_floats(None if mix is None else [c for row in mix for c in row], n * n, "hyper_residual_rms_norm mix")
+    import ctypes as _ct
+    mixa = _host_floats(mix if mix is None or isinstance(mix, _ct.Array) else [c for row in mix for c in row], n * n,
+                        "hyper_residual_rms_norm mix")
     outa = _host_floats(out_coef, n, "hyper_residual_rms_norm out_coef")
     ina = _host_floats(in_coef, n, "hyper_residual_rms_norm in_coef")
     out = torch.empty(T, W, dtype=adt, device=x.device) if want_out else None

@@ -81,12 +81,12 @@ class StreamCoefficients(nn.Module):
         self.write = nn.Parameter(torch.ones(streams, dtype=torch.float32), requires_grad=False)
         self.mix = nn.Parameter(torch.eye(streams, dtype=torch.float32), requires_grad=False)
         self.scale = nn.Parameter(torch.ones(width, dtype=dtype), requires_grad=False)
-        self.reads: Optional[List[float]] = None
+        self.reads = None
         self.wrote = None
 
     def finalize(self) -> None:
-        self.reads = self.read.tolist()
-        self.wrote = (self.mix.tolist(), self.write.tolist(), self.scale)
+        self.reads = mops.host_floats(self.read.tolist())
+        self.wrote = (mops.host_floats(self.mix.tolist()), mops.host_floats(self.write.tolist()), self.scale)
 
 
 class PagulixLayer(nn.Module):

@@ -99,7 +99,7 @@ def parse_args():
                     help="instead of the default workload: a Fatudra stack (biased attention + decay memory + mLSTM layers) beside a "
                          "Llama stack of equal size, bf16, prefill (--mixers-prompt tokens) and decode (--batch x --ctx), and every "
                          "mixer kernel alone against its roofline (aphrodite_engine_amd/bench_mixers.py); one JSON line of its own")
-    ap.add_argument("--mixers-design", default="fatudra", choices=["fatudra", "gipozen", "fekotar"],
+    ap.add_argument("--mixers-design", default="fatudra", choices=["fatudra", "gipozen", "fekotar", "pagulix"],
                     help="with --mixers: which stack stands beside Llama (gipozen: windowed differential attention with short "
                          "convolutions, depth-averaged residual, PolyNorm and routed-expert feed-forwards)")
     ap.add_argument("--mixers-prompt", type=int, default=4096)
