@@ -472,7 +472,7 @@ def pagulix_config(s):
                                            "scale": s["dim"] ** -0.5, "v_mix": True}}
     layers = [dict(l, mlp=moe) for l in (delta, latent, attn, attn)][:LAYERS]
     return {"architecture": "Pagulix", "vocab": VOCAB, "width": s["width"], "norm": {"eps": 1e-6}, "streams": PAG_STREAMS,
-            "residual_mult": 0.3, "logit_softcap": 30.0, "layers": layers}
+            "residual_mult": 0.5, "logit_softcap": 30.0, "layers": layers}
 
 
 def pagulix_kernel_section(s, prompt_len, batch, ctx, device):
@@ -511,7 +511,7 @@ def pagulix_kernel_section(s, prompt_len, batch, ctx, device):
         y, ls, w16 = torch.randn(T, W, device=device, dtype=bf), torch.randn(W, device=device, dtype=bf), torch.randn(W, device=device, dtype=bf)
         mix = (torch.eye(n) + 0.1 * torch.randn(n, n)).tolist()
         oc, ic = [1.0] * n, [0.5] * n
-        sec = timed(lambda: mops.hyper_residual_rms_norm(x, y, ls, mix, oc, 0.3, ic, w16, 1e-6))
+        sec = timed(lambda: mops.hyper_residual_rms_norm(x, y, ls, mix, oc, 0.5, ic, w16, 1e-6))
         x16, r16 = torch.randn(T, W, device=device, dtype=bf), torch.randn(T, W, device=device, dtype=bf)
         lsec = timed(lambda: ops.fused_add_rms_norm(x16, r16, w16, 1e-5))
         rec("hyper_residual_rms_norm_" + name, sec, bytes_=T * W * (8 * n + 4),

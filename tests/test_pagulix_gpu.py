@@ -291,7 +291,7 @@ LA_SHAPES = [(3, 48, 8, {"base": 5000.0, "dims": 8}), (5, 128, 32, {"base": 100.
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", LA_SHAPES)
-@pytest.mark.parametrize("window", [0, 1, 13, 40, 100])
+@pytest.mark.parametrize("window", [0, 1, 13, 45, 100])
 def test_latent_attention_window_and_sink_in_portions_and_decoded(mops, dtype, shape, window):
     H, R, P, rot = shape
     rng = np.random.default_rng(R + window)
@@ -372,7 +372,7 @@ def test_decoded_rows_under_a_window_beside_long_ones(mops):
 # ---------------------------------------------------------------------------------------------------------------------
 # router and experts
 # ---------------------------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("experts,top", [(6, 2), (8, 4), (130, 7), (5, 5), (3, 1), (70, 66)])
+@pytest.mark.parametrize("experts,top", [(6, 2), (9, 4), (130, 7), (5, 5), (3, 1), (70, 66)])
 def test_router_softmax_over_the_chosen_logits(mops, experts, top):
     rng = np.random.default_rng(experts)
     z = np.float32(rng.standard_normal((37, experts)) * 3)
@@ -430,11 +430,11 @@ CONFIGS = {
     "mixed": lambda: U.make_config([A(v_mix=False, heads=4, kv_heads=4, dim=16, vdim=24, rot_dims=16, scaling=None, mlp=None), D(), L(),
                                     A(), D(heads=3, kv_heads=3, dim=16, vdim=24, conv=2, mlp=U.moe(32, 4, 1, 0)),
                                     A(rot_dims=24, base=50.0, scaling=(2.0, 2.0, 8.0, 32)), L(heads=2, dim=16, rot_dim=12, vdim=24, kv_rank=36,
-                                                                                             window=40, mlp=None), A()]),
+                                                                                             window=44, mlp=None), A()]),
     # sizes the matrix-core kernels serve in bfloat16; one stream, no layer scale surprises, no soft cap
     "wide": lambda: U.make_config([L(heads=5, dim=24, rot_dim=32, vdim=40, kv_rank=128, window=50, mlp=U.moe(64, 4, 2, 64)),
                                    D(heads=4, kv_heads=2, dim=64, vdim=64, conv=4, mlp=U.moe(64, 8, 3, 0)),
-                                   A(heads=4, kv_heads=2, dim=64, vdim=64, rot_dims=32, v_mix=False), A(heads=8, kv_heads=2, dim=128, vdim=32, rot_dims=64)],
+                                   A(heads=4, kv_heads=2, dim=64, vdim=64, rot_dims=32, v_mix=False), A(heads=6, kv_heads=3, dim=128, vdim=64, rot_dims=32)],
                                   width=128, vocab=211, streams=1, residual_mult=1.0, softcap=0.0),
     # a window longer than anything it sees, five taps, one head
     "plain": lambda: U.make_config([D(heads=1, kv_heads=1, dim=40, vdim=20, conv=5), L(heads=1, dim=32, rot_dim=16, vdim=32, kv_rank=32, window=4000),
