@@ -504,8 +504,8 @@ class StreamedResidual:
     def start(self, table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
         """x fp32 [T, streams, W]: every stream is the embedding."""
         x = torch.empty(ids.shape[0], self.streams, table.shape[1], dtype=torch.float32, device=table.device)
-        first = mops.embed_scale(table, ids, 1.0)
-        x.copy_(first.unsqueeze(1).expand_as(x))
+        rows = ids if self.streams == 1 else ids.repeat_interleave(self.streams)       # row t * streams + s is token t
+        mops.embed_scale(table, rows, 1.0, out=x.view(-1, table.shape[1]))
         return x
 
     def step(self, x: torch.Tensor, y: Optional[torch.Tensor], wrote, reads, weight: Optional[torch.Tensor], want_sum: bool = False):
