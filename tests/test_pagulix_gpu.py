@@ -213,7 +213,8 @@ ROT_P = {"base": 100.0, "dims": 40}
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d,e,rot,layout", [(6, 2, 24, 16, ROT_S, "half"), (2, 2, 40, 72, ROT_P, "interleaved"), (3, 1, 130, 8, ROT_P, "half")])
+@pytest.mark.parametrize("H,G,d,e,rot,layout", [(6, 2, 24, 16, ROT_S, "half"), (2, 2, 40, 72, ROT_P, "interleaved"), (3, 1, 130, 8, ROT_P, "half"),
+                                                (4, 2, 64, 32, {"base": 100.0, "dims": 32}, "half")])
 @pytest.mark.parametrize("norm,blend", [(True, True), (False, False)])
 def test_rotation_norm_blend_and_cache_write(mops, dtype, H, G, d, e, rot, layout, norm, blend):
     from aphrodite_engine_amd.mixers import RotaryFrequencies
